@@ -1,0 +1,31 @@
+// C entry points of the gfx950 kernel library.  Every function launches on the
+// given stream, allocates nothing, and returns 0 or a negative code with a
+// message behind pae_last_error().  dtype codes: 0 float32, 1 bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+extern "C" {
+const char* pae_last_error();
+int pae_device_arch(char* out, int cap);  // "gfx950" on the card the kernels are built for
+
+int pae_embedding(int dtype, void* out, const void* table, const int* ids, int num_tokens, int hidden,
+                  int vocab, hipStream_t stream);
+int pae_add_rmsnorm(int dtype, void* residual, const void* delta, const void* weight, int w_is_f32, float eps,
+                    const int* rows, void* out, int num_rows, int hidden, int write_residual,
+                    hipStream_t stream);
+int pae_residual_add(int dtype, void* residual, const void* delta, int64_t n, hipStream_t stream);
+int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int rot,
+                      const float* inv_freq, const int* positions, const int* tok_seq, const int* block_tables,
+                      int max_blocks, int bs, void* k_cache, void* v_cache, int write_kv, hipStream_t stream);
+int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, hipStream_t stream);
+int pae_gemm_plain(int in_dtype, int out_dtype, void* C, int64_t ldc, const void* A, int64_t lda, const void* W,
+                   const void* bias, int b_is_f32, int M, int N, int K, hipStream_t stream);
+int pae_paged_attention_generic(int dtype, void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                const void* k_cache, const void* v_cache, const int* positions,
+                                const int* tok_seq, const int* block_tables, int max_blocks, int bs,
+                                int num_tokens, int nh, int nkv, int hd, float scale, int window,
+                                hipStream_t stream);
+int pae_sample(int* tokens, const float* logits, int64_t ld, const float* temperature, const float* uniform,
+               int num_rows, int vocab, hipStream_t stream);
+}

@@ -1,0 +1,217 @@
+// Row-wise kernels around the matrix products: embedding gather, residual add
+// fused with RMS normalisation, rotary position encoding fused with the write of
+// keys and values into their cache pages, and the SiLU gate of the feed-forward.
+//
+// The residual stream is float32 in both precisions; T is the storage type of
+// activations that feed matrix products (float or bfloat16).  Sums of squares,
+// rotation angles and the gate are computed in float32 and rounded once.
+#include "common.h"
+#include "api.h"
+
+// ---------------------------------------------------------------- embedding
+// out[t, :] = table[ids[t], :]  (engine/model.py:401,448 of the reference: a plain
+// row gather, no scaling)
+template <typename T>
+__global__ void embedding_kernel(float* __restrict__ out, const T* __restrict__ table,
+                                 const int* __restrict__ ids, int hidden) {
+  const int t = blockIdx.x;
+  const T* row = table + (int64_t)ids[t] * hidden;
+  float* dst = out + (int64_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(row[i]);
+}
+
+extern "C" int pae_embedding(int dtype, void* out, const void* table, const int* ids, int num_tokens,
+                             int hidden, int vocab, hipStream_t stream) {
+  PAE_REQUIRE(num_tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes T=%d H=%d V=%d",
+              num_tokens, hidden, vocab);
+  if (num_tokens == 0) return 0;
+  if (dtype == PAE_F32)
+    embedding_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)out, (const float*)table, ids, hidden);
+  else if (dtype == PAE_BF16)
+    embedding_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((float*)out, (const bf16_t*)table, ids, hidden);
+  else
+    return pae_fail("embedding: unknown dtype code %d", dtype);
+  return pae_check_launch("embedding");
+}
+
+// ---------------------------------------------------------------- add + RMSNorm
+// r = residual[row] (+ delta[row]);  residual[row] = r if write_residual;
+// out[b] = weight * T(r * rsqrt(mean(r^2) + eps))
+// The normalised value is rounded to T before the weight multiply, as the
+// reference does (engine/model.py:117-123: float32 inside, cast back, then scale).
+// With `rows` given, block b reads source row rows[b] (gather of selected rows).
+template <typename T, int NT>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                   const void* __restrict__ weight, int w_is_f32, float eps,
+                                   const int* __restrict__ rows, T* __restrict__ out, int hidden,
+                                   int write_residual) {
+  __shared__ float scratch[NT / PAE_WAVE];
+  const int b = blockIdx.x;
+  const int64_t src = rows ? rows[b] : b;
+  float* res = residual + src * hidden;
+  const T* del = delta ? delta + src * hidden : nullptr;
+  T* dst = out + (int64_t)b * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += NT) {
+    float r = res[i];
+    if (del) r += to_f32(del[i]);
+    if (write_residual && del) res[i] = r;
+    ss += r * r;
+  }
+  const float total = block_sum<NT / PAE_WAVE>(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += NT) {
+    float r = res[i];
+    if (del && !write_residual) r += to_f32(del[i]);
+    const float normed = round_to<T>(r * inv);
+    dst[i] = from_f32<T>(load_param(weight, w_is_f32, i) * normed);
+  }
+}
+
+extern "C" int pae_add_rmsnorm(int dtype, void* residual, const void* delta, const void* weight,
+                               int w_is_f32, float eps, const int* rows, void* out, int num_rows,
+                               int hidden, int write_residual, hipStream_t stream) {
+  PAE_REQUIRE(num_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d H=%d", num_rows, hidden);
+  PAE_REQUIRE(!(rows && write_residual), "add_rmsnorm: a row gather may not write the residual back");
+  if (num_rows == 0) return 0;
+  if (dtype == PAE_F32)
+    add_rmsnorm_kernel<float, 256><<<num_rows, 256, 0, stream>>>(
+        (float*)residual, (const float*)delta, weight, w_is_f32, eps, rows, (float*)out, hidden, write_residual);
+  else if (dtype == PAE_BF16)
+    add_rmsnorm_kernel<bf16_t, 256><<<num_rows, 256, 0, stream>>>(
+        (float*)residual, (const bf16_t*)delta, weight, w_is_f32, eps, rows, (bf16_t*)out, hidden, write_residual);
+  else
+    return pae_fail("add_rmsnorm: unknown dtype code %d", dtype);
+  return pae_check_launch("add_rmsnorm");
+}
+
+// ---------------------------------------------------------------- residual add alone
+// residual += delta (used when a block's output is needed without a following norm)
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ residual, const T* __restrict__ delta, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) residual[i] += to_f32(delta[i]);
+}
+
+extern "C" int pae_residual_add(int dtype, void* residual, const void* delta, int64_t n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dtype == PAE_F32)
+    residual_add_kernel<float><<<blocks, 256, 0, stream>>>((float*)residual, (const float*)delta, n);
+  else if (dtype == PAE_BF16)
+    residual_add_kernel<bf16_t><<<blocks, 256, 0, stream>>>((float*)residual, (const bf16_t*)delta, n);
+  else
+    return pae_fail("residual_add: unknown dtype code %d", dtype);
+  return pae_check_launch("residual_add");
+}
+
+// ---------------------------------------------------------------- rotation + cache write
+// qkv row t holds [q heads | k heads | v heads], each head `hd` wide.  Query and
+// key heads are rotated over their first `rot` features in pairs (i, i + rot/2):
+//   out[i]         = x[i] * cos - x[i + rot/2] * sin
+//   out[i + rot/2] = x[i + rot/2] * cos + x[i] * sin
+// with angle = position * inv_freq[i] in float32 (engine/model.py:126-161 of the
+// reference; rotation after the bias, before the cache write, so the cache holds
+// rotated keys and raw values).  Queries are rotated in place; keys and values
+// go to slot block_table[seq][pos / bs] * bs + pos % bs of the cache
+// (engine/attention.py:374-385,409-410), laid out [block][kv head][bs][hd].
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, int nh, int nkv, int hd,
+                                     int rot, const float* __restrict__ inv_freq,
+                                     const int* __restrict__ positions, const int* __restrict__ tok_seq,
+                                     const int* __restrict__ block_tables, int max_blocks, int bs,
+                                     T* __restrict__ k_cache, T* __restrict__ v_cache, int write_kv) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  T* row = qkv + (int64_t)t * row_stride;
+  T* q = row;
+  T* k = row + (int64_t)nh * hd;
+  T* v = k + (int64_t)nkv * hd;
+  int64_t slot_base = 0;  // element offset of (block, kv head 0, offset, 0)
+  int64_t head_step = (int64_t)bs * hd;
+  if (write_kv) {
+    const int blk = block_tables[(int64_t)tok_seq[t] * max_blocks + pos / bs];
+    slot_base = ((int64_t)blk * nkv * bs + (pos % bs)) * hd;
+  }
+  const int half = rot / 2;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float s = 0.f, c = 1.f;
+    if (inv_freq) sincosf((float)pos * inv_freq[i], &s, &c);
+    for (int h = 0; h < nh; ++h) {
+      const float a = to_f32(q[h * hd + i]), b = to_f32(q[h * hd + i + half]);
+      q[h * hd + i] = from_f32<T>(a * c - b * s);
+      q[h * hd + i + half] = from_f32<T>(b * c + a * s);
+    }
+    if (write_kv) {
+      for (int h = 0; h < nkv; ++h) {
+        const float a = to_f32(k[h * hd + i]), b = to_f32(k[h * hd + i + half]);
+        T* dst = k_cache + slot_base + h * head_step;
+        dst[i] = from_f32<T>(a * c - b * s);
+        dst[i + half] = from_f32<T>(b * c + a * s);
+      }
+    }
+  }
+  if (write_kv) {
+    const int tail = hd - rot;  // features of a key beyond the rotated ones pass through
+    for (int idx = threadIdx.x; idx < nkv * tail; idx += blockDim.x) {
+      const int h = idx / tail, i = rot + idx % tail;
+      k_cache[slot_base + h * head_step + i] = k[h * hd + i];
+    }
+    for (int idx = threadIdx.x; idx < nkv * hd; idx += blockDim.x) {
+      const int h = idx / hd, i = idx % hd;
+      v_cache[slot_base + h * head_step + i] = v[h * hd + i];
+    }
+  }
+}
+
+extern "C" int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv,
+                                 int hd, int rot, const float* inv_freq, const int* positions,
+                                 const int* tok_seq, const int* block_tables, int max_blocks, int bs,
+                                 void* k_cache, void* v_cache, int write_kv, hipStream_t stream) {
+  PAE_REQUIRE(nh > 0 && nkv >= 0 && hd > 0, "rope_kv_write: bad head sizes nh=%d nkv=%d hd=%d", nh, nkv, hd);
+  PAE_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rot, hd);
+  PAE_REQUIRE(row_stride >= (int64_t)(nh + 2 * nkv) * hd, "rope_kv_write: row stride %lld too small", (long long)row_stride);
+  PAE_REQUIRE(!write_kv || (bs > 0 && max_blocks > 0 && k_cache && v_cache && block_tables && tok_seq),
+              "rope_kv_write: cache write needs tables and pools");
+  if (num_tokens <= 0) return 0;
+  if (dtype == PAE_F32)
+    rope_kv_write_kernel<float><<<num_tokens, 128, 0, stream>>>(
+        (float*)qkv, row_stride, nh, nkv, hd, rot, inv_freq, positions, tok_seq, block_tables, max_blocks, bs,
+        (float*)k_cache, (float*)v_cache, write_kv);
+  else if (dtype == PAE_BF16)
+    rope_kv_write_kernel<bf16_t><<<num_tokens, 128, 0, stream>>>(
+        (bf16_t*)qkv, row_stride, nh, nkv, hd, rot, inv_freq, positions, tok_seq, block_tables, max_blocks, bs,
+        (bf16_t*)k_cache, (bf16_t*)v_cache, write_kv);
+  else
+    return pae_fail("rope_kv_write: unknown dtype code %d", dtype);
+  return pae_check_launch("rope_kv_write");
+}
+
+// ---------------------------------------------------------------- SiLU gate
+// out[t, j] = silu(x[t, j]) * x[t, inter + j],  silu(g) = g * sigmoid(g)
+// (engine/model.py:317-320 of the reference; gate and up are the two halves of
+// one fused projection here)
+template <typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ x, int inter, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t t = idx / inter;
+  const int j = (int)(idx % inter);
+  const float g = to_f32(x[t * 2 * inter + j]);
+  const float u = to_f32(x[t * 2 * inter + inter + j]);
+  out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, hipStream_t stream) {
+  PAE_REQUIRE(num_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", num_tokens, inter);
+  const int64_t total = (int64_t)num_tokens * inter;
+  if (total == 0) return 0;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == PAE_F32)
+    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)x, inter, total);
+  else if (dtype == PAE_BF16)
+    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, inter, total);
+  else
+    return pae_fail("swiglu: unknown dtype code %d", dtype);
+  return pae_check_launch("swiglu");
+}

@@ -1,0 +1,123 @@
+"""A model built from a plan: embedding, the scheduled blocks, final norm, head.
+
+One body serves every way of calling it, as `_run_layers` does in the reference
+(engine/model.py:322-351): embedding gather (:401,448), each scheduled block,
+final norm (:351), selection of the wanted rows and the head product without
+bias (:406,453-455).  The reference norms every row and then selects; the norm
+is row-wise, so selecting first gives the same rows.  Logits are float32 in both
+precisions.  `forward_pass_count` counts traversals of the schedule, the
+reference's proof that a step is one pass (:180-186,338).
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Mapping, Optional, Tuple
+
+import torch
+
+from .. import models as _models  # noqa: F401  (registers the architectures)
+from ..cache.manager import CacheManager
+from ..config.model_config import ModelPlan
+from ..config.registry import read_config
+from ..kernels import lib as K
+from ..parts import ResidualStream, StepContext, build_block, build_part
+from ..parts.base import NORMS
+from ..parts.linear import Linear
+from ..weights.loader import load_weights
+
+TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+def _blocks_of(plan: ModelPlan, dtype, device):
+    return [build_block(spec, dtype, device) for spec in plan.layers]
+
+
+def expected_tensors(plan: ModelPlan) -> Dict[str, Tuple[int, ...]]:
+    """Every checkpoint tensor the plan's parts declare, name -> shape."""
+    out: Dict[str, Tuple[int, ...]] = {plan.embedding_name: (plan.vocab_size, plan.hidden_size)}
+    for block in _blocks_of(plan, torch.float32, "meta"):
+        out.update(block.tensors())
+    out.update(build_part(NORMS, "norm", plan.final_norm, torch.float32, "meta").tensors(plan.final_norm_prefix))
+    if plan.head_name is not None:
+        out[plan.head_name] = (plan.vocab_size, plan.hidden_size)
+    return out
+
+
+class Model:
+    def __init__(self, plan: ModelPlan, dtype: torch.dtype, device: str = "cuda:0") -> None:
+        self.plan = plan
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.blocks = _blocks_of(plan, dtype, self.device)
+        self.final_norm = build_part(NORMS, "norm", plan.final_norm, dtype, self.device)
+        self.embedding: Optional[torch.Tensor] = None
+        self.head: Optional[Linear] = None
+        self.forward_pass_count = 0
+
+    # ------------------------------------------------------------------ weights
+    def expected_tensors(self) -> Dict[str, Tuple[int, ...]]:
+        return expected_tensors(self.plan)
+
+    def optional_tensors(self) -> Tuple[str, ...]:
+        # a file of a model with a tied head may still store the head
+        return ("lm_head.weight",) if self.plan.head_name is None else ()
+
+    def bind(self, weights: Mapping[str, torch.Tensor]) -> None:
+        plan = self.plan
+        embedding = weights[plan.embedding_name]
+        self.embedding = embedding.to(device=self.device, dtype=self.dtype).contiguous()
+        for block in self.blocks:
+            block.bind(weights)
+        self.final_norm.bind(plan.final_norm_prefix, weights)
+        if plan.head_name is None:
+            self.head = Linear(self.embedding)  # tied: the same buffer, no second copy
+        else:
+            self.head = Linear(weights[plan.head_name].to(device=self.device, dtype=self.dtype).contiguous())
+
+    # ------------------------------------------------------------------ cache needs
+    def cache_specs(self):
+        """(paged, states): per schedule stop, what it keeps per token / per request."""
+        paged, states = [], []
+        for entry in self.plan.schedule:
+            mixer = self.blocks[entry.layer].mixer
+            borrowed = entry.cache_from is not None
+            paged.append(None if borrowed else mixer.paged_spec())
+            states.append(None if borrowed else mixer.state_spec())
+        return paged, states
+
+    def new_cache(self, block_size: int, num_blocks, num_slots: int) -> CacheManager:
+        paged, states = self.cache_specs()
+        return CacheManager(paged, states, block_size, num_blocks, num_slots, self.dtype, str(self.device))
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, ctx: StepContext, token_ids: torch.Tensor, logit_rows: torch.Tensor) -> torch.Tensor:
+        """Run `token_ids` (int32 [T]) through the schedule once; float32 logits
+        [len(logit_rows), vocab] at the flat rows `logit_rows` (int32)."""
+        self.forward_pass_count += 1
+        plan = self.plan
+        residual = torch.empty((ctx.num_tokens, plan.hidden_size), dtype=torch.float32, device=self.device)
+        K.embedding(residual, self.embedding, token_ids)
+        stream = ResidualStream(residual)
+        for index, entry in enumerate(plan.schedule):
+            ctx.entry = index
+            ctx.cache_entry = index if entry.cache_from is None else entry.cache_from
+            ctx.writes_cache = entry.cache_from is None
+            self.blocks[entry.layer].forward(ctx, stream)
+        rows = logit_rows.numel()
+        if rows == 0:
+            return torch.empty((0, plan.vocab_size), dtype=torch.float32, device=self.device)
+        last = self.final_norm.forward(stream, logit_rows)
+        return self.head(last, out_dtype=torch.float32)
+
+
+def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") -> Model:
+    """The model of a folder with config.json and safetensors weights; the class
+    of model is chosen by config.json's `architectures`."""
+    if dtype not in TORCH_DTYPE:
+        raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
+    config = read_config(model_dir)
+    model = Model(config.plan(), TORCH_DTYPE[dtype], device)
+    model.config = config
+    weights = load_weights(model_dir, model.expected_tensors(), model.optional_tensors())
+    model.bind(weights)
+    return model

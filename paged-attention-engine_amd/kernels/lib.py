@@ -1,0 +1,232 @@
+"""ctypes bindings of the gfx950 kernel library and thin, checked wrappers.
+
+Every wrapper takes torch tensors that already live on the GPU, checks on the
+host that shapes and dtypes match what the kernel and its grid assume, launches
+on torch's current stream and raises `KernelError` with the library's message
+on refusal.  There is no fallback: without the library or without a GPU these
+functions raise.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from typing import Optional
+
+import torch
+
+from .build import ensure_built
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def library():
+    """The loaded kernel library (built at the first call if necessary)."""
+    global _lib
+    if _lib is None:
+        path = ensure_built()
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as err:
+            raise KernelError(f"cannot load the kernel library {path}: {err}") from err
+        _declare(lib)
+        _lib = lib
+    return _lib
+
+
+def loaded_library_path() -> Optional[str]:
+    return getattr(_lib, "_name", None) if _lib is not None else None
+
+
+def _declare(lib) -> None:
+    lib.pae_last_error.restype = c_char_p
+    P, I, L, F = c_void_p, c_int, c_int64, c_float
+    sig = {
+        "pae_device_arch": [c_char_p, I],
+        "pae_embedding": [I, P, P, P, I, I, I, P],
+        "pae_add_rmsnorm": [I, P, P, P, I, F, P, P, I, I, I, P],
+        "pae_residual_add": [I, P, P, L, P],
+        "pae_rope_kv_write": [I, P, L, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P],
+        "pae_swiglu": [I, P, P, I, I, P],
+        "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
+        "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
+        "pae_sample": [P, P, L, P, P, I, I, P],
+    }
+    for name, args in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = c_int
+
+
+def _check(code: int) -> None:
+    if code != 0:
+        raise KernelError(library().pae_last_error().decode("utf-8", "replace"))
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def code_of(dtype: torch.dtype) -> int:
+    try:
+        return _CODE[dtype]
+    except KeyError:
+        raise KernelError(f"dtype {dtype} is not one the kernels take (float32, bfloat16)") from None
+
+
+def _gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernel operands must live on the GPU; there is no CPU path")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _param(t: Optional[torch.Tensor]):
+    """(pointer, is_f32) of a vector parameter stored in float32 or bfloat16."""
+    if t is None:
+        return None, 0
+    if t.dtype not in _CODE:
+        raise KernelError(f"parameter dtype {t.dtype} not supported")
+    return t.data_ptr(), 1 if t.dtype == torch.float32 else 0
+
+
+def device_arch() -> str:
+    buf = ctypes.create_string_buffer(64)
+    _check(library().pae_device_arch(buf, 64))
+    return buf.value.decode().split(":")[0]
+
+
+def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+    """out[t] = table[ids[t]] as float32; ids int32 (checked against the table by the caller)."""
+    _gpu(out, table, ids)
+    T, H = out.shape
+    assert out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous()
+    assert ids.dtype == torch.int32 and ids.numel() == T and table.shape[1] == H
+    _check(library().pae_embedding(code_of(table.dtype), out.data_ptr(), table.data_ptr(), ids.data_ptr(),
+                                   T, H, table.shape[0], _stream()))
+
+
+def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None, write_residual: bool = True) -> None:
+    """residual (+= delta); out = weight * round(residual * rsqrt(mean(residual^2) + eps)).
+
+    With `rows` (int32), out[b] comes from source row rows[b] and nothing is written back."""
+    _gpu(residual, delta, weight, out, rows)
+    H = residual.shape[-1]
+    n = out.shape[0]
+    assert residual.dtype == torch.float32 and residual.is_contiguous() and out.is_contiguous()
+    assert out.shape[-1] == H and weight.numel() == H
+    if delta is not None:
+        assert delta.dtype == out.dtype and delta.shape == residual.shape and delta.is_contiguous()
+    if rows is None:
+        assert residual.shape[0] == n
+    else:
+        assert rows.dtype == torch.int32 and rows.numel() == n
+        write_residual = False
+    wp, wf = _param(weight)
+    _check(library().pae_add_rmsnorm(code_of(out.dtype), residual.data_ptr(), _ptr(delta), wp, wf, float(eps),
+                                     _ptr(rows), out.data_ptr(), n, H, 1 if write_residual else 0, _stream()))
+
+
+def residual_add(residual: torch.Tensor, delta: torch.Tensor) -> None:
+    _gpu(residual, delta)
+    assert residual.dtype == torch.float32 and residual.shape == delta.shape
+    assert residual.is_contiguous() and delta.is_contiguous()
+    _check(library().pae_residual_add(code_of(delta.dtype), residual.data_ptr(), delta.data_ptr(),
+                                      residual.numel(), _stream()))
+
+
+def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, inv_freq: Optional[torch.Tensor],
+                  positions: torch.Tensor, tok_seq: Optional[torch.Tensor], block_tables: Optional[torch.Tensor],
+                  block_size: int, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor]) -> None:
+    """Rotate the query heads of `qkv` in place; rotate the key heads and copy the
+    value heads into their cache slots (skipped when `k_cache` is None: then the
+    row holds query heads only and nkv must be 0)."""
+    _gpu(qkv, inv_freq, positions, tok_seq, block_tables, k_cache, v_cache)
+    T = qkv.shape[0]
+    assert qkv.dim() == 2 and qkv.stride(1) == 1 and positions.dtype == torch.int32 and positions.numel() == T
+    write = k_cache is not None
+    if inv_freq is not None:
+        assert inv_freq.dtype == torch.float32 and inv_freq.numel() == rot // 2
+    max_blocks = 0
+    if write:
+        assert v_cache is not None and k_cache.dtype == qkv.dtype == v_cache.dtype
+        assert tok_seq.dtype == torch.int32 and tok_seq.numel() == T
+        assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+        # pool layout [block][kv head][block_size][head_dim]
+        assert tuple(k_cache.shape[1:]) == (nkv, block_size, hd) and k_cache.is_contiguous()
+        assert v_cache.shape == k_cache.shape and v_cache.is_contiguous()
+        max_blocks = block_tables.shape[1]
+    _check(library().pae_rope_kv_write(code_of(qkv.dtype), qkv.data_ptr(), qkv.stride(0), T, nh, nkv, hd, rot,
+                                       _ptr(inv_freq), positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables),
+                                       max_blocks, block_size, _ptr(k_cache), _ptr(v_cache), 1 if write else 0,
+                                       _stream()))
+
+
+def swiglu(out: torch.Tensor, x: torch.Tensor) -> None:
+    """out[t, j] = silu(x[t, j]) * x[t, I + j] for x of width 2 I."""
+    _gpu(out, x)
+    T, I = out.shape
+    assert x.shape == (T, 2 * I) and x.dtype == out.dtype and x.is_contiguous() and out.is_contiguous()
+    _check(library().pae_swiglu(code_of(x.dtype), out.data_ptr(), x.data_ptr(), T, I, _stream()))
+
+
+def gemm_plain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:
+    """out[M, N] = a[M, K] @ w[N, K]^T (+ bias), float32 accumulation in k order."""
+    _gpu(out, a, w, bias)
+    M, K = a.shape
+    N = w.shape[0]
+    assert w.shape == (N, K) and w.is_contiguous() and w.dtype == a.dtype
+    assert out.shape == (M, N) and a.stride(1) == 1 and out.stride(1) == 1
+    if bias is not None:
+        assert bias.numel() == N
+    bp, bf = _param(bias)
+    _check(library().pae_gemm_plain(code_of(a.dtype), code_of(out.dtype), out.data_ptr(), out.stride(0),
+                                    a.data_ptr(), a.stride(0), w.data_ptr(), bp, bf, M, N, K, _stream()))
+
+
+def paged_attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                            positions: torch.Tensor, tok_seq: torch.Tensor, block_tables: torch.Tensor,
+                            nh: int, nkv: int, hd: int, scale: float, window: int) -> None:
+    """out[t, h*hd:(h+1)*hd] = attention of query head h of token t over the cached
+    keys start..positions[t] of sequence tok_seq[t]."""
+    _gpu(out, q, k_cache, v_cache, positions, tok_seq, block_tables)
+    T = q.shape[0]
+    bs = k_cache.shape[2]
+    assert q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nh * hd and q.dtype == k_cache.dtype == out.dtype
+    assert out.shape[0] == T and out.stride(1) == 1 and out.shape[1] >= nh * hd
+    assert tuple(k_cache.shape[1:]) == (nkv, bs, hd) and k_cache.is_contiguous()
+    assert v_cache.shape == k_cache.shape and v_cache.is_contiguous()
+    assert positions.dtype == torch.int32 and positions.numel() == T
+    assert tok_seq.dtype == torch.int32 and tok_seq.numel() == T
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    _check(library().pae_paged_attention_generic(
+        code_of(q.dtype), out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(),
+        v_cache.data_ptr(), positions.data_ptr(), tok_seq.data_ptr(), block_tables.data_ptr(),
+        block_tables.shape[1], bs, T, nh, nkv, hd, float(scale), int(window), _stream()))
+
+
+def sample(tokens: torch.Tensor, logits: torch.Tensor, temperature: Optional[torch.Tensor],
+           uniform: Optional[torch.Tensor]) -> None:
+    """tokens[r] = argmax(logits[r]) where temperature[r] == 0 (or no temperatures
+    are given), else the inverse-CDF sample of softmax(logits[r] / temperature[r]) at uniform[r]."""
+    _gpu(tokens, logits, temperature, uniform)
+    R, V = logits.shape
+    assert logits.dtype == torch.float32 and logits.stride(1) == 1
+    assert tokens.dtype == torch.int32 and tokens.numel() == R
+    for t in (temperature, uniform):
+        if t is not None:
+            assert t.dtype == torch.float32 and t.numel() == R
+    _check(library().pae_sample(tokens.data_ptr(), logits.data_ptr(), logits.stride(0), _ptr(temperature),
+                                _ptr(uniform), R, V, _stream()))

@@ -1,0 +1,133 @@
+"""What a part is, what it sees of a step, and the registries parts are found in.
+
+A model is put together from five kinds of parts, each chosen by the `kind` of
+its spec and none aware of the model it sits in:
+
+  norm               forward(stream, rows=None) -> normalised activations
+  position encoding  encode_and_store(ctx, qkv, ...): rotates queries/keys, writes the cache
+  mixer              forward(ctx, x) -> y        (attention here; may keep paged or per-request state)
+  feed-forward       forward(ctx, x) -> y
+  block              forward(ctx, stream)        (arranges two norms, a mixer and a feed-forward)
+
+Each part declares the tensors it needs (`tensors(prefix)`: name -> shape) and
+takes them in `bind(prefix, weights)`.  The reference wires the same pieces by
+hand inside one class (engine/model.py:281-351) and lets its attention backends
+vary behind `attend(layer, q, k, v)` (engine/attention.py:248-277); the registry
+and the spec-driven construction are this engine's own.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Mapping, Optional, Tuple
+
+import torch
+
+
+class ResidualStream:
+    """The float32 residual sum of a step and the branch output not yet added to it.
+
+    Norm parts add `pending` while they normalise, so the sum is formed in
+    32-bit and written once."""
+
+    def __init__(self, residual: torch.Tensor) -> None:
+        self.residual = residual
+        self.pending: Optional[torch.Tensor] = None
+
+
+@dataclass
+class StepContext:
+    """One step as parts see it: flat tokens of several sequences and their caches."""
+
+    dtype: torch.dtype                 # storage type of activations that feed matrix products
+    device: torch.device
+    num_tokens: int
+    num_seqs: int
+    positions: torch.Tensor            # int32 [T] position of each token in its sequence
+    tok_seq: torch.Tensor              # int32 [T] row of each token's sequence in the tables below
+    block_tables: Dict[int, torch.Tensor]  # cache group -> int32 [S, max_blocks]
+    slots: torch.Tensor                # int32 [S] state slot of each sequence
+    cache: "object"                    # the CacheManager
+    # the same on the host, for parts that loop over sequences
+    seq_ids: List[int] = field(default_factory=list)
+    q_starts: List[int] = field(default_factory=list)   # first flat row of each sequence
+    q_lens: List[int] = field(default_factory=list)     # rows of each sequence in this step
+    past_lens: List[int] = field(default_factory=list)  # tokens each sequence held before the step
+    host_slots: List[int] = field(default_factory=list)
+    # set by the model for the stop that is running
+    entry: int = 0                     # index in the schedule
+    cache_entry: int = 0               # the stop whose cache is read (entry itself unless it borrows)
+    writes_cache: bool = True
+
+
+class Part:
+    """Base of all parts: holds its spec and the precision it computes in."""
+
+    def __init__(self, spec, dtype: torch.dtype, device) -> None:
+        self.spec = spec
+        self.dtype = dtype
+        self.device = device
+
+    def tensors(self, prefix: str) -> Dict[str, Tuple[int, ...]]:
+        """Checkpoint tensors this part needs, by full name."""
+        return {}
+
+    def bind(self, prefix: str, weights: Mapping[str, torch.Tensor]) -> None:
+        """Take the tensors declared by `tensors(prefix)` out of `weights`."""
+
+    def matrix(self, t: torch.Tensor) -> torch.Tensor:
+        """A matrix-product operand in the compute precision, on the device."""
+        return t.to(device=self.device, dtype=self.dtype).contiguous()
+
+    def vector(self, t: torch.Tensor) -> torch.Tensor:
+        """A norm weight or bias: stays float32 if stored so, else the compute precision."""
+        keep = torch.float32 if t.dtype == torch.float32 else self.dtype
+        return t.to(device=self.device, dtype=keep).contiguous()
+
+    # what the part keeps in the cache (mixers override)
+    def paged_spec(self):
+        return None
+
+    def state_spec(self):
+        return None
+
+
+# kind -> class, one registry per role
+NORMS: Dict[str, Callable] = {}
+POSITION_ENCODINGS: Dict[str, Callable] = {}
+MIXERS: Dict[str, Callable] = {}
+FEED_FORWARDS: Dict[str, Callable] = {}
+BLOCKS: Dict[str, Callable] = {}
+
+
+def _register(table: Dict[str, Callable], kind: str):
+    def wrap(cls):
+        table[kind] = cls
+        return cls
+    return wrap
+
+
+def register_norm(kind: str):
+    return _register(NORMS, kind)
+
+
+def register_position_encoding(kind: str):
+    return _register(POSITION_ENCODINGS, kind)
+
+
+def register_mixer(kind: str):
+    return _register(MIXERS, kind)
+
+
+def register_feed_forward(kind: str):
+    return _register(FEED_FORWARDS, kind)
+
+
+def register_block(kind: str):
+    return _register(BLOCKS, kind)
+
+
+def build_part(table: Dict[str, Callable], role: str, spec, dtype, device):
+    if spec.kind not in table:
+        raise KeyError(f"no {role} of kind '{spec.kind}' is registered; known: {', '.join(sorted(table))}")
+    return table[spec.kind](spec, dtype, device)

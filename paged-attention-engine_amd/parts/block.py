@@ -1,0 +1,48 @@
+"""Arrangements of a layer's parts.
+
+"prenorm" is the reference's block (engine/model.py:340-349):
+h = h + mixer(norm1(h)); h = h + feed_forward(norm2(h)).  Each branch's output is
+left pending on the stream and added by the next norm, in float32.
+"""
+
+from __future__ import annotations
+
+from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Part, ResidualStream, build_part, register_block)
+
+
+@register_block("prenorm")
+class PreNormBlock:
+    def __init__(self, layer_spec, dtype, device):
+        self.spec = layer_spec
+        self.mixer_norm = build_part(NORMS, "norm", layer_spec.mixer_norm, dtype, device)
+        self.mixer = build_part(MIXERS, "mixer", layer_spec.mixer, dtype, device)
+        self.feed_forward_norm = build_part(NORMS, "norm", layer_spec.feed_forward_norm, dtype, device)
+        self.feed_forward = build_part(FEED_FORWARDS, "feed-forward", layer_spec.feed_forward, dtype, device)
+
+    def _named(self):
+        s = self.spec
+        return ((self.mixer_norm, s.prefix + s.mixer_norm_prefix), (self.mixer, s.prefix + s.mixer_prefix),
+                (self.feed_forward_norm, s.prefix + s.feed_forward_norm_prefix),
+                (self.feed_forward, s.prefix + s.feed_forward_prefix))
+
+    def tensors(self):
+        out = {}
+        for part, prefix in self._named():
+            out.update(part.tensors(prefix))
+        return out
+
+    def bind(self, weights):
+        for part, prefix in self._named():
+            part.bind(prefix, weights)
+
+    def forward(self, ctx, stream: ResidualStream) -> None:
+        x = self.mixer_norm.forward(stream)
+        stream.pending = self.mixer.forward(ctx, x)
+        x = self.feed_forward_norm.forward(stream)
+        stream.pending = self.feed_forward.forward(ctx, x)
+
+
+def build_block(layer_spec, dtype, device):
+    if layer_spec.arrangement not in BLOCKS:
+        raise KeyError(f"no block arrangement '{layer_spec.arrangement}'; known: {', '.join(sorted(BLOCKS))}")
+    return BLOCKS[layer_spec.arrangement](layer_spec, dtype, device)

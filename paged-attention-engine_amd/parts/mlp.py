@@ -1,0 +1,36 @@
+"""Dense gated feed-forward: down(silu(gate(x)) * up(x)), no biases
+(engine/model.py:317-320 of the reference).  gate and up are one product over
+concatenated weights; the gate is applied in float32 and rounded once."""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import lib as K
+from .base import Part, register_feed_forward
+from .linear import Linear
+
+
+@register_feed_forward("swiglu")
+class SwiGLU(Part):
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.activation != "silu":
+            raise ValueError(f"activation '{spec.activation}' is not supported by the gated feed-forward")
+
+    def tensors(self, prefix):
+        s = self.spec
+        return {prefix + "gate_proj.weight": (s.intermediate_size, s.hidden_size),
+                prefix + "up_proj.weight": (s.intermediate_size, s.hidden_size),
+                prefix + "down_proj.weight": (s.hidden_size, s.intermediate_size)}
+
+    def bind(self, prefix, weights):
+        gate_up = torch.cat([weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]], dim=0)
+        self.gate_up = Linear(self.matrix(gate_up))
+        self.down = Linear(self.matrix(weights[prefix + "down_proj.weight"]))
+
+    def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
+        both = self.gate_up(x)
+        act = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
+        K.swiglu(act, both)
+        return self.down(act)

@@ -1,0 +1,36 @@
+"""RMS normalisation fused with the pending residual add.
+
+Formula of the reference (engine/model.py:117-123): variance and scaling in
+float32, the result cast to the activation type and then multiplied by the
+weight.  The residual sum itself stays float32 here (the reference adds in the
+activation type, engine/model.py:343,349).
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import lib as K
+from .base import Part, ResidualStream, register_norm
+
+
+@register_norm("rmsnorm")
+class RMSNorm(Part):
+    def tensors(self, prefix):
+        return {prefix + "weight": (self.spec.size,)}
+
+    def bind(self, prefix, weights):
+        self.weight = self.vector(weights[prefix + "weight"])
+
+    def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Add the pending branch output into the residual and return the normalised
+        rows.  With `rows` (int32 indices) only those rows are produced and the
+        stream is left untouched."""
+        n = stream.residual.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.spec.size), dtype=self.dtype, device=stream.residual.device)
+        K.add_rmsnorm(stream.residual, stream.pending, self.weight, self.spec.eps, out, rows)
+        if rows is None:
+            stream.pending = None
+        return out

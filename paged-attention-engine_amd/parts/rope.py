@@ -1,0 +1,43 @@
+"""Rotary position encoding (pairs (i, i + rot/2)), fused with the cache write.
+
+inv_freq[i] = 1 / theta ** (2 i / rot), built exactly as the reference builds it
+(engine/model.py:132-135: int64 arange -> float, divided by the size, theta to
+that power, in float32); angle = position * inv_freq in float32
+(engine/model.py:138-152); out = x * cos + rotate_half(x) * sin (:126-129,155-161).
+The reference casts cos and sin to the activation type before the multiply; here
+they stay float32 and the result is rounded once.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import lib as K
+from .base import Part, register_position_encoding
+
+
+@register_position_encoding("neox_rope")
+class NeoxRope(Part):
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        rot = spec.rotary_dim
+        if rot % 2:
+            raise ValueError(f"rotary_dim {rot} must be even")
+        exponent = torch.arange(0, rot, 2, dtype=torch.int64).to(torch.float32)
+        self.inv_freq = (1.0 / (spec.theta ** (exponent / rot))).to(device)
+
+    def encode_and_store(self, ctx, qkv, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
+        """Rotate the query heads of `qkv` in place; write rotated keys and raw
+        values to the cache (when `k_cache` is given)."""
+        K.rope_kv_write(qkv, nh, nkv, hd, self.spec.rotary_dim, self.inv_freq, ctx.positions, ctx.tok_seq,
+                        block_table, block_size, k_cache, v_cache)
+
+
+@register_position_encoding("none")
+class NoPosition(Part):
+    """No encoding: keys and values go to the cache as they are."""
+
+    def encode_and_store(self, ctx, qkv, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
+        if k_cache is not None:
+            K.rope_kv_write(qkv, nh, nkv, hd, 0, None, ctx.positions, ctx.tok_seq, block_table, block_size,
+                            k_cache, v_cache)

@@ -1,0 +1,67 @@
+"""Random weights: a model folder (config.json, model.safetensors) from a config and a seed.
+
+The reference has this only in its tests (tests/tiny_model.py:21-50:
+`torch.manual_seed(seed)`, every matrix randn * 0.02, zero biases, unit norm
+weights).  Here biases are drawn as well, so that the bias path carries signal,
+and norm weights may be spread around 1.  Values are drawn in float32 and stored
+as bfloat16, the precision checkpoints of this family ship in, so that the
+32-bit and the bfloat16 paths start from the same numbers.
+
+Every tensor has a generator of its own, seeded from (seed, name): any tensor
+can be produced alone, on the CPU or on the device that will hold it.
+"""
+
+from __future__ import annotations
+
+import json
+import os
+import zlib
+from typing import Dict, Mapping, Tuple
+
+import torch
+
+from .safetensors_io import save_file
+
+
+def _tensor_seed(seed: int, name: str) -> int:
+    return (int(seed) * 1000003 + zlib.crc32(name.encode("utf-8"))) & 0x7FFFFFFFFFFFFFFF
+
+
+def is_norm_weight(name: str) -> bool:
+    return name.endswith("norm.weight") or name.endswith("layernorm.weight")
+
+
+def random_tensor(name: str, shape: Tuple[int, ...], seed: int, std: float = 0.02,
+                  norm_std: float = 0.0, device: str = "cpu",
+                  dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    gen = torch.Generator(device=device).manual_seed(_tensor_seed(seed, name))
+    if is_norm_weight(name):
+        t = torch.ones(shape, device=device)
+        if norm_std:
+            t += norm_std * torch.randn(shape, generator=gen, device=device)
+    else:
+        t = torch.randn(shape, generator=gen, device=device)
+        t *= std
+    return t.to(dtype)
+
+
+def random_weights(expected: Mapping[str, Tuple[int, ...]], seed: int, std: float = 0.02,
+                   norm_std: float = 0.0, device: str = "cpu",
+                   dtype: torch.dtype = torch.bfloat16) -> Dict[str, torch.Tensor]:
+    return {name: random_tensor(name, tuple(shape), seed, std, norm_std, device, dtype)
+            for name, shape in expected.items()}
+
+
+def write_model_folder(config, seed: int, out_dir: str, std: float = 0.02, norm_std: float = 0.0,
+                       dtype: torch.dtype = torch.bfloat16) -> str:
+    """Write `config.json` and `model.safetensors` for the typed `config` (any
+    registered architecture's config object) with random weights."""
+    from ..engine.model import expected_tensors  # late: parts register on import
+
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(out_dir, "config.json"), "w", encoding="utf-8") as handle:
+        json.dump(config.to_json_dict(), handle, indent=2)
+    tensors = random_weights(expected_tensors(config.plan()), seed, std, norm_std, "cpu", dtype)
+    save_file(tensors, os.path.join(out_dir, "model.safetensors"),
+              {"format": "pt", "seed": str(seed), "std": str(std), "norm_std": str(norm_std)})
+    return out_dir
