@@ -345,8 +345,9 @@ class Scheduler:
                         continue  # it was its own victim
                 self._plan(seq, count)
 
-        # 2. admission from the head of the queue: strict arrival order, no backfilling
-        while self.waiting:
+        # 2. admission from the head of the queue: strict arrival order, no backfilling;
+        #    a step that had to evict admits nobody (the pages it freed are spoken for)
+        while self.waiting and not preempted:
             head = self.waiting[0]
             if self.max_num_seqs is not None and len(self.running) >= self.max_num_seqs:
                 break
