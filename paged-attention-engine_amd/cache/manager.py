@@ -14,8 +14,10 @@ window has passed them (`release_passed`).  A reservation takes pages in every
 group or in none (the reference's all-or-nothing `append_tokens`,
 engine/cache.py:238-257, carried over to several pools).
 
-Pool layout of one group: [entry][K|V][block][kv head][block_size][head_dim], so
-that the keys of one (block, head) are one contiguous tile.
+Pool layout of one group: [entry][K|V][block][kv head][block_size * head_dim]; the
+keys of one (block, head) are one contiguous tile [block_size][head_dim], the
+values one contiguous tile stored transposed, [head_dim][block_size], which is
+what the attention kernels' matrix-core operands want.
 """
 
 from __future__ import annotations
@@ -138,10 +140,11 @@ class CacheManager:
         return None if hit is None else hit[0]
 
     def kv_of(self, entry: int) -> Tuple[torch.Tensor, torch.Tensor]:
-        """(keys, values) pools of a stop, each [block][kv head][block_size][head_dim]."""
+        """(keys, values) pools of a stop: keys [block][kv head][block_size][head_dim],
+        values [block][kv head][head_dim][block_size]."""
         g, i = self._group_of_entry[entry]
         pool = self.groups[g].pool
-        return pool[i, 0], pool[i, 1]
+        return pool[i, 0], pool[i, 1].view(pool.shape[2], pool.shape[3], pool.shape[5], pool.shape[4])
 
     def state_of(self, entry: int) -> torch.Tensor:
         return self.state_tensors[entry]

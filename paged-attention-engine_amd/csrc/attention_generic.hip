@@ -69,11 +69,12 @@ __global__ void paged_attention_generic_kernel(
     for (int j = first; j <= last; ++j) {
       const float pj = p_lds[j];
       const int rj = __shfl(row, j, PAE_WAVE);
-      const T* vr = v_cache + (int64_t)rj * hd;
+      // values are transposed within a page: [block][kv head][feature][offset in page]
+      const T* vr = v_cache + (int64_t)(rj / bs) * bs * hd + rj % bs;
 #pragma unroll
       for (int i = 0; i < MAXD; ++i) {
         const int d = lane + i * PAE_WAVE;
-        if (d < hd) acc[i] = fmaf(pj, to_f32(vr[d]), acc[i]);
+        if (d < hd) acc[i] = fmaf(pj, to_f32(vr[(int64_t)d * bs]), acc[i]);
       }
     }
     __syncthreads();

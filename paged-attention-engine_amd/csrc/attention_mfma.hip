@@ -1,0 +1,359 @@
+// Causal attention over the paged cache on the matrix cores (bfloat16 in,
+// float32 scores, softmax and accumulation).
+//
+// Both kernels work on transposed tiles so that the softmax output can feed the
+// second product without leaving registers:
+//   S^T[16 keys x 16 columns] = K[16 keys x hd] * Q^T        (MFMA 16x16x32, k = hd)
+//   O^T[hd x 16 columns]     += V^T[hd x 16 keys] * P^T       (MFMA 16x16x16, k = keys)
+// The accumulator layout of S^T (lane = column, registers = 4 consecutive keys) is
+// exactly the B-operand layout of the second product.  A "column" is one (token,
+// query head); the 16 keys of a tile are one cache page (or a 16-key slice of a
+// larger page).  Keys live as [block][kv head][page][hd], values transposed as
+// [block][kv head][hd][page], so both A operands are contiguous per lane.
+//
+// decode:  one workgroup per (sequence with a single new token, kv head, split of
+//          the keys); the columns are the query heads that share the kv head, so a
+//          page is read once for all of them.  Four wavefronts take pages in turn
+//          and merge in LDS; splits are merged by a second kernel.  Splits start at
+//          multiples of the split length from position 0.
+// prefill: one wavefront per (32 consecutive tokens of a sequence, query head).
+//
+// Masking is the reference's rule (engine/attention.py:474-487: key j visible iff
+// j <= position of the query) plus an optional window.  A column's result depends
+// only on its own position: fully masked pages add exact zeros.
+#include "common.h"
+#include "api.h"
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+#define NEG_BIG (-1.0e30f)
+#define LOG2E 1.4426950408889634f
+
+__device__ __forceinline__ short bf16_bits(float x) {
+  const bf16_t h = __float2bfloat16(x);
+  return *reinterpret_cast<const short*>(&h);
+}
+
+// State of CT column tiles of one wavefront.
+template <int HD, int CT>
+struct AttnState {
+  f32x4 acc[CT][HD / 16];  // O^T: rows hd = 16 t + 4 g4 + i, column = lane % 16
+  float m[CT];             // running maximum of the column (in units of log2)
+  float l[CT];             // this lane's share of the column's sum
+};
+
+// One 16-key tile.  `kp` points at key row 0 of the tile (row stride HD), `vp` at
+// value feature 0 of the tile's first key (feature stride `vstride` elements).
+// q[ct][j]: B operand of column tile ct for hd slice j.  pos/start: per lane's column.
+template <int HD, int CT>
+__device__ __forceinline__ void attn_tile(AttnState<HD, CT>& st, const bf16x8 (&kf)[HD / 32],
+                                          const s16x4 (&vf)[HD / 16], const bf16x8 (&q)[CT][HD / 32],
+                                          int key0, const int (&pos)[CT], const int (&start)[CT],
+                                          float scale_log2) {
+  const int g4 = threadIdx.x % PAE_WAVE / 16;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < HD / 32; ++j) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j], q[ct][j], s, 0, 0, 0);
+    float mx = NEG_BIG;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = key0 + 4 * g4 + i;
+      s[i] = (key <= pos[ct] && key >= start[ct]) ? s[i] * scale_log2 : -INFINITY;
+      mx = fmaxf(mx, s[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, PAE_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, PAE_WAVE));
+    const float m_new = fmaxf(st.m[ct], mx);
+    const float alpha = exp2f(st.m[ct] - m_new);
+    st.m[ct] = m_new;
+    float psum = 0.f;
+    s16x4 pb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = exp2f(s[i] - m_new);
+      psum += p;
+      pb[i] = bf16_bits(p);
+    }
+    st.l[ct] = st.l[ct] * alpha + psum;
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) {
+      st.acc[ct][t] *= alpha;
+      st.acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[t], pb, st.acc[ct][t], 0, 0, 0);
+    }
+  }
+}
+
+template <int HD>
+__device__ __forceinline__ void load_kv_tile(bf16x8 (&kf)[HD / 32], s16x4 (&vf)[HD / 16], const bf16_t* kp,
+                                             const bf16_t* vp, int vstride) {
+  const int lane = threadIdx.x % PAE_WAVE;
+  const int r = lane % 16, g4 = lane / 16;
+#pragma unroll
+  for (int j = 0; j < HD / 32; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(kp + r * HD + 32 * j + 8 * g4);
+#pragma unroll
+  for (int t = 0; t < HD / 16; ++t)
+    vf[t] = *reinterpret_cast<const s16x4*>(vp + (int64_t)(16 * t + r) * vstride + 4 * g4);
+}
+
+// ------------------------------------------------------------------ decode
+// part_acc[(token, head, split)][hd] unnormalised, part_ml[(token, head, split)][2] = (max, sum)
+template <int HD>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int max_splits, const bf16_t* __restrict__ q,
+    int64_t q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ dec_tok, const int* __restrict__ positions, const int* __restrict__ tok_seq,
+    const int* __restrict__ block_tables, int max_blocks, int bs, int nh, int nkv, float scale_log2,
+    int window, int split_len) {
+  const int split = blockIdx.x, kvh = blockIdx.y;
+  const int tok = dec_tok[blockIdx.z];
+  const int pos[1] = {positions[tok]};
+  const int start[1] = {(window > 0 && pos[0] - window + 1 > 0) ? pos[0] - window + 1 : 0};
+  const int lo = max(split * split_len, start[0] / 16 * 16);
+  const int hi = min((split + 1) * split_len, pos[0] + 1);  // keys [lo, hi)
+  if (lo >= hi) return;
+  const int* table = block_tables + (int64_t)tok_seq[tok] * max_blocks;
+  const int g = nh / nkv;
+  const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
+  const int col = lane % 16, g4 = lane / 16;
+
+  bf16x8 qf[1][HD / 32];
+  {
+    const bf16_t* qrow = q + (int64_t)tok * q_stride + (int64_t)(kvh * g + (col < g ? col : 0)) * HD;
+#pragma unroll
+    for (int j = 0; j < HD / 32; ++j) {
+      qf[0][j] = *reinterpret_cast<const bf16x8*>(qrow + 32 * j + 8 * g4);
+      if (col >= g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[0][j][e] = (__bf16)0.f;
+    }
+  }
+  AttnState<HD, 1> st;
+  st.m[0] = NEG_BIG;
+  st.l[0] = 0.f;
+#pragma unroll
+  for (int t = 0; t < HD / 16; ++t) st.acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int page_elems = bs * HD;
+  // 16-key tiles of the split, taken by the four wavefronts in turn
+  const int tile_lo = lo / 16, tile_hi = (hi + 15) / 16;
+  bf16x8 kf[HD / 32];
+  s16x4 vf[HD / 16];
+  for (int tile = tile_lo + wave; tile < tile_hi; tile += 4) {
+    const int key0 = tile * 16;
+    const int blk = table[key0 / bs];
+    const int64_t base = ((int64_t)blk * nkv + kvh) * page_elems;
+    load_kv_tile<HD>(kf, vf, k_cache + base + (int64_t)(key0 % bs) * HD, v_cache + base + key0 % bs, bs);
+    attn_tile<HD, 1>(st, kf, vf, qf, key0, pos, start, scale_log2);
+  }
+
+  // merge wavefronts 1..3 into wavefront 0, one after the other: every lane of a
+  // wavefront holds the same (column, features) as the same lane of wavefront 0
+  extern __shared__ float s_buf[];  // [HD / 4 + 2][64]
+  for (int w = 1; w < 4; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int t = 0; t < HD / 16; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_buf[(4 * t + i) * PAE_WAVE + lane] = st.acc[0][t][i];
+      s_buf[(HD / 4) * PAE_WAVE + lane] = st.m[0];
+      s_buf[(HD / 4 + 1) * PAE_WAVE + lane] = st.l[0];
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const float mw = s_buf[(HD / 4) * PAE_WAVE + lane];
+      const float m_new = fmaxf(st.m[0], mw);
+      const float f0 = exp2f(st.m[0] - m_new), fw = exp2f(mw - m_new);
+#pragma unroll
+      for (int t = 0; t < HD / 16; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          st.acc[0][t][i] = st.acc[0][t][i] * f0 + s_buf[(4 * t + i) * PAE_WAVE + lane] * fw;
+      st.l[0] = st.l[0] * f0 + s_buf[(HD / 4 + 1) * PAE_WAVE + lane] * fw;
+      st.m[0] = m_new;
+    }
+    __syncthreads();
+  }
+  if (wave != 0) return;
+  float l = st.l[0];
+  l += __shfl_xor(l, 16, PAE_WAVE);
+  l += __shfl_xor(l, 32, PAE_WAVE);
+  if (col < g) {
+    const int64_t slot = ((int64_t)blockIdx.z * nh + kvh * g + col) * max_splits + split;
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t)
+      *reinterpret_cast<f32x4*>(part_acc + slot * HD + 16 * t + 4 * g4) = st.acc[0][t];
+    if (g4 == 0) {
+      part_ml[slot * 2] = st.m[0];
+      part_ml[slot * 2 + 1] = l;
+    }
+  }
+}
+
+// out[token, head, :] = sum over the splits that hold keys, in split order
+template <int HD>
+__global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
+                                         const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                         int max_splits, const int* __restrict__ dec_tok,
+                                         const int* __restrict__ positions, int nh, int window, int split_len) {
+  const int head = blockIdx.x;
+  const int tok = dec_tok[blockIdx.y];
+  const int pos = positions[tok];
+  const int start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first = start / split_len, last = pos / split_len;
+  const int64_t slot0 = ((int64_t)blockIdx.y * nh + head) * max_splits;
+  float m = NEG_BIG;
+  for (int s = first; s <= last; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float a = 0.f, l = 0.f;
+    for (int s = first; s <= last; ++s) {
+      const float f = exp2f(part_ml[(slot0 + s) * 2] - m);
+      a += f * part_acc[(slot0 + s) * HD + d];
+      l += f * part_ml[(slot0 + s) * 2 + 1];
+    }
+    out[(int64_t)tok * out_stride + (int64_t)head * HD + d] = __float2bfloat16(a / l);
+  }
+}
+
+// ------------------------------------------------------------------ prefill
+// tiles[t] = (row of the sequence in the tables, first flat token, number of tokens <= 32);
+// the tokens of a tile are consecutive in the step and in position.
+#define PREFILL_CT 2
+template <int HD>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ tiles,
+    int num_tiles, const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks,
+    int bs, int nh, int nkv, float scale_log2, int window) {
+  const int wave = threadIdx.x / PAE_WAVE, lane = threadIdx.x % PAE_WAVE;
+  const int tile_id = blockIdx.x * 4 + wave;
+  if (tile_id >= num_tiles) return;
+  const int head = blockIdx.y;
+  const int kvh = head / (nh / nkv);
+  const int seq_row = tiles[tile_id * 3], tok0 = tiles[tile_id * 3 + 1], ntok = tiles[tile_id * 3 + 2];
+  const int* table = block_tables + (int64_t)seq_row * max_blocks;
+  const int col = lane % 16, g4 = lane / 16;
+  const int pos0 = positions[tok0];
+
+  int pos[PREFILL_CT], start[PREFILL_CT];
+  bf16x8 qf[PREFILL_CT][HD / 32];
+  int lo = pos0, hi = pos0;  // keys any column needs: [lo, hi]
+#pragma unroll
+  for (int ct = 0; ct < PREFILL_CT; ++ct) {
+    const int c = ct * 16 + col;
+    const bool live = c < ntok;
+    pos[ct] = live ? pos0 + c : -1;  // a dead column sees no key
+    start[ct] = (live && window > 0 && pos[ct] - window + 1 > 0) ? pos[ct] - window + 1 : 0;
+    const bf16_t* qrow = q + (int64_t)(tok0 + (live ? c : 0)) * q_stride + (int64_t)head * HD;
+#pragma unroll
+    for (int j = 0; j < HD / 32; ++j) qf[ct][j] = *reinterpret_cast<const bf16x8*>(qrow + 32 * j + 8 * g4);
+  }
+  hi = pos0 + ntok - 1;
+  lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+
+  AttnState<HD, PREFILL_CT> st;
+#pragma unroll
+  for (int ct = 0; ct < PREFILL_CT; ++ct) {
+    st.m[ct] = NEG_BIG;
+    st.l[ct] = 0.f;
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) st.acc[ct][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  const int page_elems = bs * HD;
+  bf16x8 kf[HD / 32];
+  s16x4 vf[HD / 16];
+  for (int key0 = lo / 16 * 16; key0 <= hi; key0 += 16) {
+    const int blk = table[key0 / bs];
+    const int64_t base = ((int64_t)blk * nkv + kvh) * page_elems;
+    load_kv_tile<HD>(kf, vf, k_cache + base + (int64_t)(key0 % bs) * HD, v_cache + base + key0 % bs, bs);
+    attn_tile<HD, PREFILL_CT>(st, kf, vf, qf, key0, pos, start, scale_log2);
+  }
+#pragma unroll
+  for (int ct = 0; ct < PREFILL_CT; ++ct) {
+    float l = st.l[ct];
+    l += __shfl_xor(l, 16, PAE_WAVE);
+    l += __shfl_xor(l, 32, PAE_WAVE);
+    const int c = ct * 16 + col;
+    if (c >= ntok) continue;
+    const float inv = 1.0f / l;
+    bf16_t* o = out + (int64_t)(tok0 + c) * out_stride + (int64_t)head * HD;
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) {
+      s16x4 w;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] = bf16_bits(st.acc[ct][t][i] * inv);
+      *reinterpret_cast<s16x4*>(o + 16 * t + 4 * g4) = w;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ entry points
+#define FOR_HEAD_DIM(hd, CALL)                                       \
+  switch (hd) {                                                      \
+    case 32: { CALL(32); break; }                                    \
+    case 64: { CALL(64); break; }                                    \
+    case 96: { CALL(96); break; }                                    \
+    case 128: { CALL(128); break; }                                  \
+    case 160: { CALL(160); break; }                                  \
+    case 192: { CALL(192); break; }                                  \
+    case 224: { CALL(224); break; }                                  \
+    case 256: { CALL(256); break; }                                  \
+    default: return pae_fail("matrix-core attention takes head_dim in multiples of 32 up to 256, got %d", hd); \
+  }
+
+static int check_common(const char* what, int nh, int nkv, int hd, int bs, int max_blocks, int window) {
+  PAE_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "%s: %d query heads over %d key/value heads", what, nh, nkv);
+  PAE_REQUIRE(nh / nkv <= 16, "%s: more than 16 query heads per key/value head (%d)", what, nh / nkv);
+  PAE_REQUIRE(bs >= 16 && bs % 16 == 0, "%s: page size %d is not a multiple of 16", what, bs);
+  PAE_REQUIRE(max_blocks > 0 && window >= 0, "%s: bad table width %d or window %d", what, max_blocks, window);
+  PAE_REQUIRE(hd % 32 == 0 && hd >= 32 && hd <= 256, "%s: head_dim %d is not a multiple of 32 up to 256", what, hd);
+  return 0;
+}
+
+// Workspace: part_acc holds num_dec * nh * max_splits * hd floats, part_ml num_dec * nh * max_splits * 2.
+extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                    const void* k_cache, const void* v_cache, const int* dec_tok, int num_dec,
+                                    const int* positions, const int* tok_seq, const int* block_tables,
+                                    int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
+                                    int split_len, void* part_acc, void* part_ml, hipStream_t stream) {
+  if (int rc = check_common("attn_decode", nh, nkv, hd, bs, max_blocks, window)) return rc;
+  PAE_REQUIRE(split_len >= 64 && split_len % 64 == 0, "attn_decode: split length %d is not a multiple of 64", split_len);
+  PAE_REQUIRE(num_dec <= 65535 && nkv <= 65535, "attn_decode: grid too large");
+  if (num_dec <= 0) return 0;
+  const int max_splits = (int)(((int64_t)max_blocks * bs + split_len - 1) / split_len);
+  const float scale_log2 = scale * LOG2E;
+  dim3 grid(max_splits, nkv, num_dec), merge_grid(nh, num_dec);
+#define CALL(HD)                                                                                              \
+  attn_decode_kernel<HD><<<grid, 256, (size_t)(HD / 4 + 2) * PAE_WAVE * sizeof(float), stream>>>(                         \
+      (float*)part_acc, (float*)part_ml, max_splits, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,      \
+      (const bf16_t*)v_cache, dec_tok, positions, tok_seq, block_tables, max_blocks, bs, nh, nkv, scale_log2, \
+      window, split_len);                                                                                     \
+  attn_decode_merge_kernel<HD><<<merge_grid, 64, 0, stream>>>((bf16_t*)out, out_stride, (const float*)part_acc, \
+                                                              (const float*)part_ml, max_splits, dec_tok,     \
+                                                              positions, nh, window, split_len)
+  FOR_HEAD_DIM(hd, CALL)
+#undef CALL
+  return pae_check_launch("attn_decode");
+}
+
+extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                     const void* k_cache, const void* v_cache, const int* tiles, int num_tiles,
+                                     const int* positions, const int* block_tables, int max_blocks, int bs,
+                                     int nh, int nkv, int hd, float scale, int window, hipStream_t stream) {
+  if (int rc = check_common("attn_prefill", nh, nkv, hd, bs, max_blocks, window)) return rc;
+  PAE_REQUIRE(nh <= 65535, "attn_prefill: grid too large");
+  if (num_tiles <= 0) return 0;
+  const float scale_log2 = scale * LOG2E;
+  dim3 grid((num_tiles + 3) / 4, nh);
+#define CALL(HD)                                                                                          \
+  attn_prefill_kernel<HD><<<grid, 256, 0, stream>>>((bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, \
+                                                    (const bf16_t*)k_cache, (const bf16_t*)v_cache, tiles, \
+                                                    num_tiles, positions, block_tables, max_blocks, bs, nh, \
+                                                    nkv, scale_log2, window)
+  FOR_HEAD_DIM(hd, CALL)
+#undef CALL
+  return pae_check_launch("attn_prefill");
+}

@@ -114,7 +114,8 @@ extern "C" int pae_residual_add(int dtype, void* residual, const void* delta, in
 // reference; rotation after the bias, before the cache write, so the cache holds
 // rotated keys and raw values).  Queries are rotated in place; keys and values
 // go to slot block_table[seq][pos / bs] * bs + pos % bs of the cache
-// (engine/attention.py:374-385,409-410), laid out [block][kv head][bs][hd].
+// (engine/attention.py:374-385,409-410); keys are laid out [block][kv head][bs][hd],
+// values transposed within the page, [block][kv head][hd][bs].
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, int nh, int nkv, int hd,
                                      int rot, const float* __restrict__ inv_freq,
@@ -127,12 +128,11 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, in
   T* q = row;
   T* k = row + (int64_t)nh * hd;
   T* v = k + (int64_t)nkv * hd;
-  int64_t slot_base = 0;  // element offset of (block, kv head 0, offset, 0)
-  int64_t head_step = (int64_t)bs * hd;
-  if (write_kv) {
-    const int blk = block_tables[(int64_t)tok_seq[t] * max_blocks + pos / bs];
-    slot_base = ((int64_t)blk * nkv * bs + (pos % bs)) * hd;
-  }
+  int64_t page_base = 0;  // element offset of (block, kv head 0) in either pool
+  const int64_t head_step = (int64_t)bs * hd;
+  const int off = pos % bs;
+  if (write_kv) page_base = (int64_t)block_tables[(int64_t)tok_seq[t] * max_blocks + pos / bs] * nkv * head_step;
+  const int64_t slot_base = page_base + (int64_t)off * hd;  // key row of this token, kv head 0
   const int half = rot / 2;
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     float s = 0.f, c = 1.f;
@@ -157,9 +157,11 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, in
       const int h = idx / tail, i = rot + idx % tail;
       k_cache[slot_base + h * head_step + i] = k[h * hd + i];
     }
+    // values are stored transposed within a page: [kv head][feature][offset in page]
+    const int64_t v_base = page_base + off;
     for (int idx = threadIdx.x; idx < nkv * hd; idx += blockDim.x) {
       const int h = idx / hd, i = idx % hd;
-      v_cache[slot_base + h * head_step + i] = v[h * hd + i];
+      v_cache[v_base + h * head_step + (int64_t)i * bs] = v[h * hd + i];
     }
   }
 }

@@ -23,6 +23,9 @@ from ..parts import StepContext
 from .model import Model
 
 
+TILE_TOKENS = 32  # tokens per run handed to the prefill attention kernel
+
+
 @dataclass(frozen=True)
 class StepEntry:
     seq_id: int
@@ -84,9 +87,15 @@ class StepRunner:
             per_seq = [cache.block_table(group.index, s) for s in seq_ids]
             width = max(1, max(len(t) for t in per_seq))
             tables.append((width, per_seq))
-        total = 3 * T + S + len(rows) + sum(S * w for w, _ in tables)
+        decode_tokens = [q_starts[i] for i in range(S) if q_lens[i] == 1]
+        tiles: List[int] = []
+        for i in range(S):
+            if q_lens[i] > 1:
+                for first in range(0, q_lens[i], TILE_TOKENS):
+                    tiles += [i, q_starts[i] + first, min(TILE_TOKENS, q_lens[i] - first)]
+        total = 3 * T + S + len(rows) + len(decode_tokens) + len(tiles) + sum(S * w for w, _ in tables)
         staging = torch.empty(total, dtype=torch.int32, pin_memory=True)
-        flat: List[int] = ids + positions + tok_seq + slots + rows
+        flat: List[int] = ids + positions + tok_seq + slots + rows + decode_tokens + tiles
         for width, per_seq in tables:
             for table in per_seq:
                 flat.extend(table)
@@ -102,6 +111,7 @@ class StepRunner:
             return out
 
         d_ids, d_pos, d_seq, d_slots, d_rows = take(T), take(T), take(T), take(S), take(len(rows))
+        d_decode, d_tiles = take(len(decode_tokens)), take(len(tiles)).view(-1, 3)
         block_tables: Dict[int, torch.Tensor] = {}
         for group, (width, _) in zip(cache.groups, tables):
             block_tables[group.index] = take(S * width).view(S, width)
@@ -109,5 +119,6 @@ class StepRunner:
         ctx = StepContext(dtype=self.model.dtype, device=self.device, num_tokens=T, num_seqs=S,
                           positions=d_pos, tok_seq=d_seq, block_tables=block_tables, slots=d_slots,
                           cache=cache, seq_ids=seq_ids, q_starts=q_starts, q_lens=q_lens,
-                          past_lens=past_lens, host_slots=slots)
+                          past_lens=past_lens, host_slots=slots, decode_tokens=d_decode,
+                          prefill_tiles=d_tiles)
         return self.model.forward(ctx, d_ids, d_rows)

@@ -59,6 +59,8 @@ def _declare(lib) -> None:
         "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "pae_sample": [P, P, L, P, P, I, I, P],
+        "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P, P, P],
+        "pae_attn_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -99,6 +101,13 @@ def _param(t: Optional[torch.Tensor]):
     if t.dtype not in _CODE:
         raise KernelError(f"parameter dtype {t.dtype} not supported")
     return t.data_ptr(), 1 if t.dtype == torch.float32 else 0
+
+
+def _check_pools(k_cache, v_cache, nkv: int, bs: int, hd: int) -> None:
+    """Keys [block][kv head][bs][hd]; values transposed within the page, [block][kv head][hd][bs]."""
+    assert tuple(k_cache.shape[1:]) == (nkv, bs, hd) and k_cache.is_contiguous()
+    assert tuple(v_cache.shape) == (k_cache.shape[0], nkv, hd, bs) and v_cache.is_contiguous()
+    assert k_cache.dtype == v_cache.dtype
 
 
 def device_arch() -> str:
@@ -164,9 +173,7 @@ def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, inv_f
         assert v_cache is not None and k_cache.dtype == qkv.dtype == v_cache.dtype
         assert tok_seq.dtype == torch.int32 and tok_seq.numel() == T
         assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
-        # pool layout [block][kv head][block_size][head_dim]
-        assert tuple(k_cache.shape[1:]) == (nkv, block_size, hd) and k_cache.is_contiguous()
-        assert v_cache.shape == k_cache.shape and v_cache.is_contiguous()
+        _check_pools(k_cache, v_cache, nkv, block_size, hd)
         max_blocks = block_tables.shape[1]
     _check(library().pae_rope_kv_write(code_of(qkv.dtype), qkv.data_ptr(), qkv.stride(0), T, nh, nkv, hd, rot,
                                        _ptr(inv_freq), positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables),
@@ -206,8 +213,7 @@ def paged_attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.T
     bs = k_cache.shape[2]
     assert q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nh * hd and q.dtype == k_cache.dtype == out.dtype
     assert out.shape[0] == T and out.stride(1) == 1 and out.shape[1] >= nh * hd
-    assert tuple(k_cache.shape[1:]) == (nkv, bs, hd) and k_cache.is_contiguous()
-    assert v_cache.shape == k_cache.shape and v_cache.is_contiguous()
+    _check_pools(k_cache, v_cache, nkv, bs, hd)
     assert positions.dtype == torch.int32 and positions.numel() == T
     assert tok_seq.dtype == torch.int32 and tok_seq.numel() == T
     assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
@@ -215,6 +221,57 @@ def paged_attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.T
         code_of(q.dtype), out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(),
         v_cache.data_ptr(), positions.data_ptr(), tok_seq.data_ptr(), block_tables.data_ptr(),
         block_tables.shape[1], bs, T, nh, nkv, hd, float(scale), int(window), _stream()))
+
+
+DECODE_SPLIT = 256  # keys per workgroup of the decode kernel; fixed, so results do not depend on the batch
+
+
+def mfma_attention_supported(dtype: torch.dtype, nh: int, nkv: int, hd: int, bs: int) -> bool:
+    """Shapes the matrix-core attention kernels take; others go through the generic kernel."""
+    return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 256 and bs % 16 == 0 and nh // nkv <= 16
+
+
+def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                dec_tok: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
+                block_tables: torch.Tensor, nh: int, nkv: int, hd: int, scale: float, window: int) -> None:
+    """Attention of the single new token of each sequence listed in `dec_tok` (flat
+    token indices) over that sequence's cached keys: split over the keys, then merged."""
+    _gpu(out, q, k_cache, v_cache, dec_tok, positions, tok_seq, block_tables)
+    n = dec_tok.numel()
+    bs = k_cache.shape[2]
+    assert q.dtype == torch.bfloat16 == out.dtype == k_cache.dtype and q.stride(1) == 1 and out.stride(1) == 1
+    assert q.shape[1] >= nh * hd and out.shape[1] >= nh * hd and out.shape[0] == q.shape[0]
+    _check_pools(k_cache, v_cache, nkv, bs, hd)
+    assert dec_tok.dtype == torch.int32 and positions.dtype == torch.int32 and tok_seq.dtype == torch.int32
+    assert positions.numel() == q.shape[0] == tok_seq.numel()
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    max_splits = -(-block_tables.shape[1] * bs // DECODE_SPLIT)
+    part_acc = torch.empty((n * nh * max_splits, hd), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((n * nh * max_splits, 2), dtype=torch.float32, device=q.device)
+    _check(library().pae_attn_decode_bf16(
+        out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+        dec_tok.data_ptr(), n, positions.data_ptr(), tok_seq.data_ptr(), block_tables.data_ptr(),
+        block_tables.shape[1], bs, nh, nkv, hd, float(scale), int(window), DECODE_SPLIT,
+        part_acc.data_ptr(), part_ml.data_ptr(), _stream()))
+
+
+def attn_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                 tiles: torch.Tensor, positions: torch.Tensor, block_tables: torch.Tensor,
+                 nh: int, nkv: int, hd: int, scale: float, window: int) -> None:
+    """Attention of runs of up to 32 consecutive tokens; tiles[t] = (table row of the
+    sequence, first flat token, number of tokens)."""
+    _gpu(out, q, k_cache, v_cache, tiles, positions, block_tables)
+    bs = k_cache.shape[2]
+    assert q.dtype == torch.bfloat16 == out.dtype == k_cache.dtype and q.stride(1) == 1 and out.stride(1) == 1
+    assert q.shape[1] >= nh * hd and out.shape[1] >= nh * hd and out.shape[0] == q.shape[0]
+    _check_pools(k_cache, v_cache, nkv, bs, hd)
+    assert tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.is_contiguous()
+    assert positions.dtype == torch.int32 and positions.numel() == q.shape[0]
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    _check(library().pae_attn_prefill_bf16(
+        out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+        tiles.data_ptr(), tiles.shape[0], positions.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
+        bs, nh, nkv, hd, float(scale), int(window), _stream()))
 
 
 def sample(tokens: torch.Tensor, logits: torch.Tensor, temperature: Optional[torch.Tensor],

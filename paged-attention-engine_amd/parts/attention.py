@@ -76,6 +76,14 @@ class PagedAttention(Part):
             self.position.encode_and_store(ctx, qkv, s.num_heads, 0, s.head_dim, None, None, None,
                                            ctx.cache.block_size)
         attn = torch.empty((x.shape[0], s.num_heads * s.head_dim), dtype=x.dtype, device=x.device)
-        K.paged_attention_generic(attn, qkv, k_cache, v_cache, ctx.positions, ctx.tok_seq, table,
-                                  s.num_heads, s.num_kv_heads, s.head_dim, s.scale, s.window or 0)
+        geometry = (s.num_heads, s.num_kv_heads, s.head_dim, s.scale, s.window or 0)
+        if K.mfma_attention_supported(x.dtype, s.num_heads, s.num_kv_heads, s.head_dim, ctx.cache.block_size) \
+                and ctx.decode_tokens is not None:
+            if ctx.decode_tokens.numel():
+                K.attn_decode(attn, qkv, k_cache, v_cache, ctx.decode_tokens, ctx.positions, ctx.tok_seq, table,
+                              *geometry)
+            if ctx.prefill_tiles.numel():
+                K.attn_prefill(attn, qkv, k_cache, v_cache, ctx.prefill_tiles, ctx.positions, table, *geometry)
+        else:
+            K.paged_attention_generic(attn, qkv, k_cache, v_cache, ctx.positions, ctx.tok_seq, table, *geometry)
         return self.out(attn)

@@ -1,0 +1,294 @@
+"""Each kernel alone against a plain PyTorch float32/float64 reference of the same
+op, at sizes other than the engine's tiny models (odd widths, other head sizes
+and group sizes, larger pages, fragmented block tables).  Where random inputs
+would hide a fault, one score is made to stand out."""
+
+import math
+
+import pytest
+import torch
+
+from tests.plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def K():
+    from paged_attention_engine_amd.kernels import lib
+    return lib
+
+
+def tol(dtype, scale=1.0):
+    return (2e-6 if dtype == "float32" else 2.0 ** -7) * scale
+
+
+# ------------------------------------------------------------------ small row-wise kernels
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embedding(dtype):
+    table = torch.randn(301, 72).to(DT[dtype])
+    ids = torch.tensor([5, 300, 0, 5, 17], dtype=torch.int32)
+    out = torch.empty(5, 72, dtype=torch.float32, device=DEV)
+    K().embedding(out, table.to(DEV), ids.to(DEV))
+    assert torch.equal(out.cpu(), table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden", [72, 1536, 1000])
+def test_add_rmsnorm(dtype, hidden):
+    torch.manual_seed(0)
+    n, eps = 7, 1e-5
+    res = torch.randn(n, hidden) * 3
+    delta = torch.randn(n, hidden).to(DT[dtype])
+    w = (1 + 0.1 * torch.randn(hidden)).to(DT[dtype])
+    summed = res + delta.float()
+    # reference: normalise in float32, round to the storage type, multiply by the weight, round
+    normed = (summed * torch.rsqrt(summed.pow(2).mean(-1, keepdim=True) + eps)).to(DT[dtype])
+    want = (w.float() * normed.float()).to(DT[dtype]).float()
+    r = res.to(DEV)
+    out = torch.empty(n, hidden, dtype=DT[dtype], device=DEV)
+    K().add_rmsnorm(r, delta.to(DEV), w.to(DEV), eps, out)
+    assert torch.allclose(r.cpu(), summed, atol=1e-6)  # the sum is formed and kept in float32
+    assert (out.float().cpu() - want).abs().max() <= tol(dtype, float(want.abs().max()))
+    # gather of selected rows: nothing is written back; a float32 weight is taken as stored
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    r2 = res.to(DEV)
+    out2 = torch.empty(3, hidden, dtype=DT[dtype], device=DEV)
+    K().add_rmsnorm(r2, delta.to(DEV), w.float().to(DEV), eps, out2, rows)
+    assert torch.equal(r2.cpu(), res)
+    assert (out2.float().cpu() - want[[6, 0, 3]]).abs().max() <= tol(dtype, float(want.abs().max()))
+    # no pending branch: plain norm of the residual; zero rows give zero, not NaN
+    r3 = torch.zeros(2, hidden, device=DEV)
+    out3 = torch.empty(2, hidden, dtype=DT[dtype], device=DEV)
+    K().add_rmsnorm(r3, None, w.to(DEV), eps, out3)
+    assert torch.equal(out3.float().cpu(), torch.zeros(2, hidden))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,N,K_", [(1, 50, 72), (70, 193, 100), (5, 1000, 353), (64, 64, 16)])
+def test_gemm_plain(dtype, M, N, K_):
+    torch.manual_seed(1)
+    a = torch.randn(M, K_).to(DT[dtype])
+    w = torch.randn(N, K_).to(DT[dtype])
+    b = torch.randn(N).to(DT[dtype])
+    want = a.double() @ w.double().t() + b.double()
+    out = torch.empty(M, N, dtype=DT[dtype], device=DEV)
+    K().gemm_plain(out, a.to(DEV), w.to(DEV), b.to(DEV))
+    assert (out.double().cpu() - want).abs().max() <= tol(dtype, float(want.abs().max())) * (4 if dtype == "float32" else 1)
+    if dtype == "bfloat16":  # float32 results from bfloat16 operands (the head's product)
+        out32 = torch.empty(M, N, dtype=torch.float32, device=DEV)
+        K().gemm_plain(out32, a.to(DEV), w.to(DEV), None)
+        assert (out32.double().cpu() - (want - b.double())).abs().max() <= 1e-5 * float(want.abs().max())
+    else:  # a row's result does not depend on the rows beside it
+        one = torch.empty(1, N, dtype=torch.float32, device=DEV)
+        K().gemm_plain(one, a[M - 1:].to(DEV), w.to(DEV), b.to(DEV))
+        assert torch.equal(one[0], out[M - 1])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_swiglu(dtype):
+    x = (torch.randn(9, 2 * 177) * 3).to(DT[dtype])
+    x[0, :5] = torch.tensor([0.0, -30.0, 30.0, -100.0, 100.0]).to(DT[dtype])
+    want = plain.silu(x[:, :177].double()) * x[:, 177:].double()
+    out = torch.empty(9, 177, dtype=DT[dtype], device=DEV)
+    K().swiglu(out, x.to(DEV))
+    assert torch.isfinite(out).all()
+    assert (out.double().cpu() - want).abs().max() <= tol(dtype, float(want.abs().max()))
+
+
+# ------------------------------------------------------------------ paged cache helpers
+def scattered_tables(seq_lens, bs, num_blocks, seed=0, width=None):
+    """Block tables drawn from a shuffled pool: descending, non-adjacent, fragmented
+    (the reference fragments its pool for the same reason, tests/test_parity.py:196-223)."""
+    gen = torch.Generator().manual_seed(seed)
+    order = torch.randperm(num_blocks, generator=gen).tolist()
+    need = [-(-n // bs) for n in seq_lens]
+    assert sum(need) <= num_blocks
+    width = width or max(need)
+    tables = torch.full((len(seq_lens), width), -1, dtype=torch.int32)
+    for s, n in enumerate(need):
+        tables[s, :n] = torch.tensor([order.pop() for _ in range(n)], dtype=torch.int32)
+    return tables
+
+
+def fill_pools(keys, values, tables, bs, num_blocks, dtype):
+    """keys/values: per sequence [n, nkv, hd].  Pools: K [nb][nkv][bs][hd], V [nb][nkv][hd][bs]."""
+    nkv, hd = keys[0].shape[1:]
+    kp = torch.zeros(num_blocks, nkv, bs, hd, dtype=dtype)
+    vp = torch.zeros(num_blocks, nkv, hd, bs, dtype=dtype)
+    for s, (k, v) in enumerate(zip(keys, values)):
+        for p in range(k.shape[0]):
+            blk = int(tables[s, p // bs])
+            kp[blk, :, p % bs, :] = k[p].to(dtype)
+            vp[blk, :, :, p % bs] = v[p].to(dtype)
+    return kp, vp
+
+
+def reference_attention(q, k, v, pos, scale, window):
+    """One query (nh, hd) at position `pos` over keys/values [n, nkv, hd] in float64."""
+    nh, nkv = q.shape[0], k.shape[1]
+    g = nh // nkv
+    start = max(0, pos - window + 1) if window else 0
+    out = torch.empty(nh, v.shape[-1], dtype=torch.float64)
+    for h in range(nh):
+        kk = k[start:pos + 1, h // g].double()
+        vv = v[start:pos + 1, h // g].double()
+        w = torch.softmax((kk @ q[h].double()) * scale, 0)
+        out[h] = w @ vv
+    return out
+
+
+# ------------------------------------------------------------------ rotation and cache write
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,rot,bs", [(4, 2, 16, 16, 4), (6, 1, 48, 48, 16), (3, 3, 32, 16, 8)])
+def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs):
+    torch.manual_seed(2)
+    theta = 50000.0
+    # two sequences: one brings positions 5..11, the other the single position 37
+    positions = list(range(5, 12)) + [37]
+    tok_seq = [0] * 7 + [1]
+    tables = scattered_tables([12, 38], bs, 40, seed=3)
+    T = len(positions)
+    qkv = torch.randn(T, (nh + 2 * nkv) * hd).to(DT[dtype])
+    inv = plain.rope_inv_freq(rot, theta)
+    kp = torch.full((40, nkv, bs, hd), 7.0, dtype=DT[dtype])
+    vp = torch.full((40, nkv, hd, bs), 7.0, dtype=DT[dtype])
+    d_qkv, d_kp, d_vp = qkv.to(DEV), kp.to(DEV), vp.to(DEV)
+    K().rope_kv_write(d_qkv, nh, nkv, hd, rot, inv.to(DEV), torch.tensor(positions, dtype=torch.int32, device=DEV),
+                      torch.tensor(tok_seq, dtype=torch.int32, device=DEV), tables.to(DEV), bs, d_kp, d_vp)
+    x = qkv.double().view(T, nh + 2 * nkv, hd)
+    cos, sin = plain.rope_cos_sin(plain.rope_inv_freq(rot, theta, torch.float64), torch.tensor(positions), torch.float64)
+    rotated = x.clone()
+    rotated[..., :rot] = x[..., :rot] * cos[:, None] + plain.rotate_half(x[..., :rot]) * sin[:, None]
+    got_q = d_qkv.cpu().double().view(T, nh + 2 * nkv, hd)[:, :nh]
+    bound = tol(dtype, 4.0) if dtype == "bfloat16" else 2e-5  # float32 angles up to 37 rad
+    assert (got_q - rotated[:, :nh]).abs().max() <= bound
+    # keys (rotated) and values (raw) sit at block_table[pos // bs] * bs + pos % bs; nothing else changed
+    want_k, want_v = kp.clone().double(), vp.clone().double()
+    for t, (p, s) in enumerate(zip(positions, tok_seq)):
+        blk = int(tables[s, p // bs])
+        want_k[blk, :, p % bs, :] = rotated[t, nh:nh + nkv]
+        want_v[blk, :, :, p % bs] = x[t, nh + nkv:]
+    assert (d_kp.cpu().double() - want_k).abs().max() <= bound
+    assert torch.equal(d_vp.cpu().double(), want_v)
+    untouched = torch.ones(40, dtype=torch.bool)
+    for p, s in zip(positions, tok_seq):
+        untouched[int(tables[s, p // bs])] = False
+    assert torch.equal(d_kp.cpu()[untouched], kp[untouched])
+
+
+# ------------------------------------------------------------------ attention
+def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=None, seed=0):
+    """Queries are the last q_lens[s] positions of each sequence.  Returns (got, want)."""
+    torch.manual_seed(seed)
+    num_blocks = sum(-(-n // bs) for n in seq_lens) + 5
+    tables = scattered_tables(seq_lens, bs, num_blocks, seed=seed + 1)
+    keys = [torch.randn(n, nkv, hd) for n in seq_lens]
+    values = [torch.randn(n, nkv, hd) for n in seq_lens]
+    positions, tok_seq = [], []
+    for s, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        positions += list(range(n - ql, n))
+        tok_seq += [s] * ql
+    T = len(positions)
+    q = torch.randn(T, nh, hd)
+    if sharp is not None:  # make one key of sequence 0 dominate its last query's scores
+        key_pos = sharp
+        direction = torch.randn(hd)
+        direction /= direction.norm()
+        keys[0][key_pos] = 6.0 * direction * math.sqrt(hd) ** 0.5
+        q[q_lens[0] - 1] = 6.0 * direction * math.sqrt(hd) ** 0.5
+    scale = hd ** -0.5
+    q, keys, values = q.to(DT[dtype]), [k.to(DT[dtype]) for k in keys], [v.to(DT[dtype]) for v in values]
+    want = torch.stack([reference_attention(q[t].float(), keys[s].float(), values[s].float(), p, scale, window)
+                        for t, (p, s) in enumerate(zip(positions, tok_seq))]).view(T, nh * hd)
+    kp, vp = fill_pools(keys, values, tables, bs, num_blocks, DT[dtype])
+    d = lambda x, dt=None: (x if dt is None else torch.tensor(x, dtype=dt)).to(DEV)
+    out = torch.zeros(T, nh * hd, dtype=DT[dtype], device=DEV)
+    qd = d(q.view(T, nh * hd).contiguous())
+    pos_d, seq_d, tab_d = d(positions, torch.int32), d(tok_seq, torch.int32), d(tables)
+    if kind == "generic":
+        K().paged_attention_generic(out, qd, d(kp), d(vp), pos_d, seq_d, tab_d, nh, nkv, hd, scale, window)
+    else:
+        starts = [sum(q_lens[:s]) for s in range(len(q_lens))]
+        dec = [starts[s] for s in range(len(q_lens)) if q_lens[s] == 1]
+        tiles = []
+        for s, ql in enumerate(q_lens):
+            if ql > 1:
+                for first in range(0, ql, 32):
+                    tiles.append([s, starts[s] + first, min(32, ql - first)])
+        if dec:
+            K().attn_decode(out, qd, d(kp), d(vp), d(dec, torch.int32), pos_d, seq_d, tab_d, nh, nkv, hd, scale, window)
+        if tiles:
+            K().attn_prefill(out, qd, d(kp), d(vp), d(tiles, torch.int32), pos_d, tab_d, nh, nkv, hd, scale, window)
+    return out.double().cpu(), want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,bs,window", [(4, 2, 16, 4, 0), (6, 2, 48, 16, 0), (7, 1, 80, 8, 0),
+                                                   (8, 8, 128, 16, 0), (6, 2, 64, 16, 37), (2, 1, 256, 32, 70)])
+def test_generic_attention(dtype, nh, nkv, hd, bs, window):
+    got, want = run_attention("generic", dtype, nh, nkv, hd, bs, window, [150, 1, 67, 330], [20, 1, 1, 75])
+    assert (got - want).abs().max() <= (1e-5 if dtype == "float32" else 3e-2)
+
+
+MFMA_SHAPES = [(12, 2, 128, 16, 0), (14, 2, 64, 16, 0), (4, 4, 32, 16, 0), (16, 1, 96, 32, 0),
+               (7, 1, 256, 16, 0), (12, 2, 128, 16, 100), (6, 3, 64, 32, 33), (5, 1, 160, 16, 0)]
+
+
+@pytest.mark.parametrize("nh,nkv,hd,bs,window", MFMA_SHAPES)
+def test_matrix_core_attention_mixed_batch(nh, nkv, hd, bs, window):
+    # decodes at an odd context, at one token, right after and right before a page's and a split's edge,
+    # beside prompt portions of 2, 33 and 150 tokens (the last one starting in the middle of a cache)
+    seq_lens = [777, 1, 257, 256, 40, 33, 600, 513]
+    q_lens = [1, 1, 1, 1, 2, 33, 150, 1]
+    got, want = run_attention("mfma", "bfloat16", nh, nkv, hd, bs, window, seq_lens, q_lens)
+    err = (got - want).abs().max(dim=1).values
+    assert float(err.max()) <= 3e-2, f"worst rows: {torch.topk(err, 5)}"
+
+
+@pytest.mark.parametrize("kind", ["generic", "mfma"])
+@pytest.mark.parametrize("key_pos,window,seen", [(3, 0, True), (255, 0, True), (256, 0, True), (700, 0, True),
+                                                  (1299, 0, True), (1299 - 63, 64, True), (1299 - 64, 64, False)])
+def test_one_far_key_stands_out(kind, key_pos, window, seen):
+    """A single key carries almost all of the last query's weight: the output is that key's value
+    if and only if the key is visible (far away among 1,300, on a page's or split's edge, at the
+    window's edge), which a kernel that drops or adds one key cannot get right."""
+    nh, nkv, hd, bs = 12, 2, 128, 16
+    got, want = run_attention(kind, "bfloat16", nh, nkv, hd, bs, window, [1300, 90], [1, 1], sharp=key_pos)
+    assert (got - want).abs().max() <= 3e-2
+    # the construction works: the visible key really dominates (else the check above says little)
+    if seen:
+        assert want[0].abs().max() > 0.5
+
+
+@pytest.mark.parametrize("q_len", [2, 31, 32, 33, 64, 100])
+def test_matrix_core_prefill_from_empty_and_warm(q_len):
+    got, want = run_attention("mfma", "bfloat16", 12, 2, 128, 16, 0, [q_len, 200 + q_len], [q_len, q_len])
+    assert (got - want).abs().max() <= 3e-2
+
+
+# ------------------------------------------------------------------ sampling
+def test_sampling_kernel():
+    torch.manual_seed(5)
+    V = 1000
+    logits = torch.randn(6, V) * 2
+    logits[1, 400] = logits[1, 17] = 9.0  # a tie: the first maximum wins
+    logits[2] = -1e9
+    logits[2, 777] = 0.0                 # one-hot
+    temps = torch.tensor([0.0, 0.0, 0.8, 0.8, 1.5, 0.3])
+    us = torch.tensor([0.3, 0.9, 0.99, 0.5, 0.123, 0.77])
+    tokens = torch.empty(6, dtype=torch.int32, device=DEV)
+    K().sample(tokens, logits.to(DEV), temps.to(DEV), us.to(DEV))
+    got = tokens.cpu().tolist()
+    want = [plain.sample_from_logits(logits[r], float(temps[r]), float(us[r])) for r in range(6)]
+    assert got == want and got[1] == 17 and got[2] == 777
+    K().sample(tokens, logits.to(DEV), None, None)
+    assert tokens.cpu().tolist() == logits.argmax(-1).tolist()
+    # a wide vocabulary that is no multiple of the block, many draws
+    V = 151_936 + 3
+    row = torch.randn(1, V) * 3
+    d_row = row.to(DEV)
+    for u in (0.0, 1e-7, 0.25, 0.5, 0.75, 0.999999):
+        K().sample(tokens[:1], d_row, torch.tensor([0.9], device=DEV), torch.tensor([u], device=DEV))
+        assert int(tokens[0]) == plain.sample_from_logits(row[0], 0.9, u)
