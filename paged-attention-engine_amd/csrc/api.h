@@ -11,16 +11,19 @@ int pae_device_arch(char* out, int cap);  // "gfx950" on the card the kernels ar
 
 int pae_embedding(int dtype, void* out, const void* table, const int* ids, int num_tokens, int hidden,
                   int vocab, hipStream_t stream);
-int pae_add_rmsnorm(int dtype, void* residual, const void* delta, const void* weight, int w_is_f32, float eps,
-                    const int* rows, void* out, int num_rows, int hidden, int write_residual,
-                    hipStream_t stream);
+int pae_add_rmsnorm(int dtype, void* residual, const void* delta, int parts, int64_t part_stride,
+                    const void* weight, int w_is_f32, float eps, const int* rows, void* out, int num_rows,
+                    int hidden, int write_residual, hipStream_t stream);
 int pae_residual_add(int dtype, void* residual, const void* delta, int64_t n, hipStream_t stream);
 int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int rot,
                       const float* inv_freq, const int* positions, const int* tok_seq, const int* block_tables,
                       int max_blocks, int bs, void* k_cache, void* v_cache, int write_kv, hipStream_t stream);
-int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, hipStream_t stream);
+int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, int block, hipStream_t stream);
 int pae_gemm_plain(int in_dtype, int out_dtype, void* C, int64_t ldc, const void* A, int64_t lda, const void* W,
                    const void* bias, int b_is_f32, int M, int N, int K, hipStream_t stream);
+int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
+                    const void* bias, int b_is_f32, int M, int N, int K, int splits, int64_t part_stride,
+                    hipStream_t stream);
 int pae_paged_attention_generic(int dtype, void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                 const void* k_cache, const void* v_cache, const int* positions,
                                 const int* tok_seq, const int* block_tables, int max_blocks, int bs,

@@ -40,46 +40,56 @@ extern "C" int pae_embedding(int dtype, void* out, const void* table, const int*
 // The normalised value is rounded to T before the weight multiply, as the
 // reference does (engine/model.py:117-123: float32 inside, cast back, then scale).
 // With `rows` given, block b reads source row rows[b] (gather of selected rows).
+// The pending branch output `delta` is either in the storage type T (parts == 0) or
+// `parts` float32 partial sums, `part_stride` elements apart, added in order.
+template <typename T>
+__device__ __forceinline__ float pending_at(const void* delta, int parts, int64_t part_stride, int64_t idx) {
+  if (parts == 0) return to_f32(((const T*)delta)[idx]);
+  float sum = 0.f;
+  for (int p = 0; p < parts; ++p) sum += ((const float*)delta)[p * part_stride + idx];
+  return sum;
+}
+
 template <typename T, int NT>
-__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
-                                   const void* __restrict__ weight, int w_is_f32, float eps,
-                                   const int* __restrict__ rows, T* __restrict__ out, int hidden,
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const void* __restrict__ delta, int parts,
+                                   int64_t part_stride, const void* __restrict__ weight, int w_is_f32,
+                                   float eps, const int* __restrict__ rows, T* __restrict__ out, int hidden,
                                    int write_residual) {
   __shared__ float scratch[NT / PAE_WAVE];
   const int b = blockIdx.x;
   const int64_t src = rows ? rows[b] : b;
   float* res = residual + src * hidden;
-  const T* del = delta ? delta + src * hidden : nullptr;
   T* dst = out + (int64_t)b * hidden;
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += NT) {
     float r = res[i];
-    if (del) r += to_f32(del[i]);
-    if (write_residual && del) res[i] = r;
+    if (delta) r += pending_at<T>(delta, parts, part_stride, src * hidden + i);
+    if (write_residual && delta) res[i] = r;
     ss += r * r;
   }
   const float total = block_sum<NT / PAE_WAVE>(ss, scratch);
   const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
   for (int i = threadIdx.x; i < hidden; i += NT) {
     float r = res[i];
-    if (del && !write_residual) r += to_f32(del[i]);
+    if (delta && !write_residual) r += pending_at<T>(delta, parts, part_stride, src * hidden + i);
     const float normed = round_to<T>(r * inv);
     dst[i] = from_f32<T>(load_param(weight, w_is_f32, i) * normed);
   }
 }
 
-extern "C" int pae_add_rmsnorm(int dtype, void* residual, const void* delta, const void* weight,
-                               int w_is_f32, float eps, const int* rows, void* out, int num_rows,
-                               int hidden, int write_residual, hipStream_t stream) {
+extern "C" int pae_add_rmsnorm(int dtype, void* residual, const void* delta, int parts, int64_t part_stride,
+                               const void* weight, int w_is_f32, float eps, const int* rows, void* out,
+                               int num_rows, int hidden, int write_residual, hipStream_t stream) {
+  PAE_REQUIRE(parts >= 0, "add_rmsnorm: negative number of partial sums");
   PAE_REQUIRE(num_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d H=%d", num_rows, hidden);
   PAE_REQUIRE(!(rows && write_residual), "add_rmsnorm: a row gather may not write the residual back");
   if (num_rows == 0) return 0;
   if (dtype == PAE_F32)
     add_rmsnorm_kernel<float, 256><<<num_rows, 256, 0, stream>>>(
-        (float*)residual, (const float*)delta, weight, w_is_f32, eps, rows, (float*)out, hidden, write_residual);
+        (float*)residual, delta, parts, part_stride, weight, w_is_f32, eps, rows, (float*)out, hidden, write_residual);
   else if (dtype == PAE_BF16)
     add_rmsnorm_kernel<bf16_t, 256><<<num_rows, 256, 0, stream>>>(
-        (float*)residual, (const bf16_t*)delta, weight, w_is_f32, eps, rows, (bf16_t*)out, hidden, write_residual);
+        (float*)residual, delta, parts, part_stride, weight, w_is_f32, eps, rows, (bf16_t*)out, hidden, write_residual);
   else
     return pae_fail("add_rmsnorm: unknown dtype code %d", dtype);
   return pae_check_launch("add_rmsnorm");
@@ -193,26 +203,32 @@ extern "C" int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int n
 // out[t, j] = silu(x[t, j]) * x[t, inter + j],  silu(g) = g * sigmoid(g)
 // (engine/model.py:317-320 of the reference; gate and up are the two halves of
 // one fused projection here)
+// With `block` > 0 the row holds blocks of `block` gate features followed by their
+// `block` up features (the layout the skinny product's gated epilogue reads).
 template <typename T>
-__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ x, int inter, int64_t total) {
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ x, int inter, int block, int64_t total) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const int64_t t = idx / inter;
   const int j = (int)(idx % inter);
-  const float g = to_f32(x[t * 2 * inter + j]);
-  const float u = to_f32(x[t * 2 * inter + inter + j]);
+  const int64_t gi = block ? (int64_t)(j / block) * 2 * block + j % block : j;
+  const int64_t ui = block ? gi + block : (int64_t)inter + j;
+  const float g = to_f32(x[t * 2 * inter + gi]);
+  const float u = to_f32(x[t * 2 * inter + ui]);
   out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
 }
 
-extern "C" int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, hipStream_t stream) {
+extern "C" int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, int block,
+                          hipStream_t stream) {
   PAE_REQUIRE(num_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", num_tokens, inter);
+  PAE_REQUIRE(block >= 0 && (block == 0 || inter % block == 0), "swiglu: blocks of %d do not divide %d", block, inter);
   const int64_t total = (int64_t)num_tokens * inter;
   if (total == 0) return 0;
   const unsigned blocks = (unsigned)((total + 255) / 256);
   if (dtype == PAE_F32)
-    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)x, inter, total);
+    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)x, inter, block, total);
   else if (dtype == PAE_BF16)
-    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, inter, total);
+    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, inter, block, total);
   else
     return pae_fail("swiglu: unknown dtype code %d", dtype);
   return pae_check_launch("swiglu");

@@ -1,0 +1,197 @@
+// C[M,N] = A[M,K] * W[N,K]^T for few rows (M <= 64): the matrix products of a
+// decode step, which are bound by reading W once from HBM.
+//
+// W (bfloat16, (out_features, in_features) row-major as in the checkpoint) is the
+// A operand of MFMA 16x16x32, 16 weight rows per tile; the activations are the B
+// operand, 16 rows of A per column tile, so each weight fragment is loaded once
+// and used for every row of A.  A workgroup owns 16 weight rows (32 for the gated
+// epilogue) and a range of k; its four wavefronts take 32-wide k steps in turn
+// and are summed in LDS in wavefront order.  With several k ranges (grid.y > 1)
+// each writes its own float32 partial, which the consumer adds up in range
+// order: no atomics, the same sums in the same order on every run.
+//
+// Epilogues: bfloat16 out with bias; float32 out (logits, or partial sums);
+// SiLU gate: rows come in blocks of 16 gate rows followed by their 16 up rows,
+// and out[m, j] = silu(gate_j) * up_j (engine/model.py:317-320 of the reference).
+#include "common.h"
+#include "api.h"
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+#define EPI_BF16 0
+#define EPI_F32 1
+#define EPI_SWIGLU 2
+#define SKINNY_U 4  // k steps of a wavefront whose loads are in flight together
+
+__device__ __forceinline__ short to_bf16_bits(float x) {
+  const bf16_t h = __float2bfloat16(x);
+  return *reinterpret_cast<const short*>(&h);
+}
+
+template <int MT, int EPI>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out, int64_t ldc,
+                                                          const bf16_t* __restrict__ A, int64_t lda,
+                                                          const bf16_t* __restrict__ W,
+                                                          const void* __restrict__ bias, int b_is_f32, int M,
+                                                          int N, int K, int k_per_split, int64_t part_stride) {
+  constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
+  __shared__ float s_part[3][RT * MT * 4][PAE_WAVE];
+  const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
+  const int r = lane % 16, g4 = lane / 16;
+  const int n0 = blockIdx.x * 16 * RT;
+  const int k_lo = blockIdx.y * k_per_split;
+  const int k_hi = min(K, k_lo + k_per_split);
+
+  const bf16_t* wrow[RT];
+  bool wok[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int n = n0 + 16 * rt + r;
+    wok[rt] = n < N;
+    wrow[rt] = W + (int64_t)(wok[rt] ? n : N - 1) * K;
+  }
+  const bf16_t* arow[MT];
+  bool aok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + r;
+    aok[mt] = m < M;
+    arow[mt] = A + (int64_t)(aok[mt] ? m : 0) * lda;
+  }
+  f32x4 acc[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  // Every lane of a wavefront runs the same number of steps (the matrix instruction
+  // takes operands from all 64 lanes).  Loads are unconditional, from clamped
+  // addresses, and issued SKINNY_U steps ahead of their use; a lane past the end of
+  // the k range zeroes its weight fragment (rows past N or M are simply not stored).
+  const bf16x8 zero = {};
+  for (int kb = k_lo + 32 * wave; kb < k_hi; kb += 128 * SKINNY_U) {
+    bf16x8 wf[SKINNY_U][RT], af[SKINNY_U][MT];
+    bool kok[SKINNY_U];
+#pragma unroll
+    for (int u = 0; u < SKINNY_U; ++u) {
+      const int k = kb + 128 * u + 8 * g4;
+      kok[u] = k < k_hi;  // K and the range bounds are multiples of 8: all 8 elements in or out
+      const int kc = k < K - 8 ? k : K - 8;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) wf[u][rt] = *reinterpret_cast<const bf16x8*>(wrow[rt] + kc);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) af[u][mt] = *reinterpret_cast<const bf16x8*>(arow[mt] + kc);
+    }
+#pragma unroll
+    for (int u = 0; u < SKINNY_U; ++u) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const bf16x8 w = kok[u] ? wf[u][rt] : zero;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, af[u][mt], acc[rt][mt], 0, 0, 0);
+      }
+    }
+  }
+
+  if (wave > 0) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_part[wave - 1][(rt * MT + mt) * 4 + i][lane] = acc[rt][mt][i];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int w = 0; w < 3; ++w)
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[rt][mt][i] += s_part[w][(rt * MT + mt) * 4 + i][lane];
+
+  const bool vec = ldc % 4 == 0;  // rows of out keep 8- and 16-byte stores aligned
+  // lane holds, per column tile mt, row m = 16 mt + r of A and weight rows 4 g4 + i of the tile
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + r;
+    if (m >= M) continue;
+    if (EPI == EPI_SWIGLU) {
+      const int j = blockIdx.x * 16 + 4 * g4;  // output feature of register 0
+      if (j >= N / 2) continue;                // N counts gate and up rows; whole blocks of 16 only
+      s16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float g = acc[0][mt][i], u = acc[1][mt][i];
+        v[i] = to_bf16_bits(g / (1.0f + expf(-g)) * u);
+      }
+      *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j) = v;
+    } else {
+      const int n = n0 + 4 * g4;
+      if (n >= N) continue;
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = acc[0][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f);
+      if (EPI == EPI_F32) {
+        float* dst = (float*)out + (int64_t)blockIdx.y * part_stride + (int64_t)m * ldc + n;
+        if (vec && n + 4 <= N) *reinterpret_cast<f32x4*>(dst) = (f32x4){v[0], v[1], v[2], v[3]};
+        else
+          for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = v[i];
+      } else {
+        bf16_t* dst = (bf16_t*)out + (int64_t)m * ldc + n;
+        if (vec && n + 4 <= N) {
+          s16x4 p;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) p[i] = to_bf16_bits(v[i]);
+          *reinterpret_cast<s16x4*>(dst) = p;
+        } else
+          for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = __float2bfloat16(v[i]);
+      }
+    }
+  }
+}
+
+// epilogue: 0 bfloat16 out (+bias), 1 float32 out (`splits` partials of `part_stride`
+// elements each when splits > 1; a bias only with one split), 2 SiLU gate (N counts the
+// interleaved gate and up rows; out is [M, N / 2]).
+extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
+                               const void* bias, int b_is_f32, int M, int N, int K, int splits,
+                               int64_t part_stride, hipStream_t stream) {
+  PAE_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d is outside 0..64", M);
+  PAE_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && lda % 8 == 0, "gemm_skinny: N=%d K=%d lda=%lld (K and lda must be multiples of 8)",
+              N, K, (long long)lda);
+  PAE_REQUIRE(splits >= 1 && (splits == 1 || epilogue == EPI_F32), "gemm_skinny: %d k ranges need the float32 epilogue", splits);
+  PAE_REQUIRE(!(bias && splits > 1), "gemm_skinny: a bias cannot be combined with partial sums");
+  PAE_REQUIRE(epilogue != EPI_SWIGLU || (N % 32 == 0 && ldc % 4 == 0), "gemm_skinny: gated epilogue needs N %% 32 == 0, got %d", N);
+  if (M == 0) return 0;
+  const int rows_per_wg = epilogue == EPI_SWIGLU ? 32 : 16;
+  int k_per_split = (K + splits - 1) / splits;
+  k_per_split = (k_per_split + 127) / 128 * 128;
+  PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "gemm_skinny: %d k ranges are too many for K=%d", splits, K);
+  dim3 grid((N + rows_per_wg - 1) / rows_per_wg, splits);
+  const int mt = (M + 15) / 16;
+#define LAUNCH(MT, EPI)                                                                                       \
+  gemm_skinny_kernel<MT, EPI><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, bias, \
+                                                        b_is_f32, M, N, K, k_per_split, part_stride)
+#define BY_MT(EPI)                       \
+  switch (mt) {                          \
+    case 1: LAUNCH(1, EPI); break;       \
+    case 2: LAUNCH(2, EPI); break;       \
+    case 3: LAUNCH(3, EPI); break;       \
+    default: LAUNCH(4, EPI); break;      \
+  }
+  switch (epilogue) {
+    case EPI_BF16: BY_MT(EPI_BF16); break;
+    case EPI_F32: BY_MT(EPI_F32); break;
+    case EPI_SWIGLU: BY_MT(EPI_SWIGLU); break;
+    default: return pae_fail("gemm_skinny: unknown epilogue %d", epilogue);
+  }
+#undef BY_MT
+#undef LAUNCH
+  return pae_check_launch("gemm_skinny");
+}

@@ -107,7 +107,7 @@ class Model:
         if rows == 0:
             return torch.empty((0, plan.vocab_size), dtype=torch.float32, device=self.device)
         last = self.final_norm.forward(stream, logit_rows)
-        return self.head(last, out_dtype=torch.float32)
+        return self.head.float32(last)
 
 
 def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") -> Model:

@@ -52,10 +52,11 @@ def _declare(lib) -> None:
     sig = {
         "pae_device_arch": [c_char_p, I],
         "pae_embedding": [I, P, P, P, I, I, I, P],
-        "pae_add_rmsnorm": [I, P, P, P, I, F, P, P, I, I, I, P],
+        "pae_add_rmsnorm": [I, P, P, I, L, P, I, F, P, P, I, I, I, P],
         "pae_residual_add": [I, P, P, L, P],
         "pae_rope_kv_write": [I, P, L, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P],
-        "pae_swiglu": [I, P, P, I, I, P],
+        "pae_swiglu": [I, P, P, I, I, I, P],
+        "pae_gemm_skinny": [I, P, L, P, L, P, P, I, I, I, I, I, L, P],
         "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "pae_sample": [P, P, L, P, P, I, I, P],
@@ -130,21 +131,30 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
                 out: torch.Tensor, rows: Optional[torch.Tensor] = None, write_residual: bool = True) -> None:
     """residual (+= delta); out = weight * round(residual * rsqrt(mean(residual^2) + eps)).
 
-    With `rows` (int32), out[b] comes from source row rows[b] and nothing is written back."""
+    `delta` is the pending branch output: [T, H] in out's dtype, or float32 partial sums
+    [P, T, H] that are added in order.  With `rows` (int32), out[b] comes from source row
+    rows[b] and nothing is written back."""
     _gpu(residual, delta, weight, out, rows)
     H = residual.shape[-1]
     n = out.shape[0]
     assert residual.dtype == torch.float32 and residual.is_contiguous() and out.is_contiguous()
     assert out.shape[-1] == H and weight.numel() == H
+    parts, part_stride = 0, 0
     if delta is not None:
-        assert delta.dtype == out.dtype and delta.shape == residual.shape and delta.is_contiguous()
+        assert delta.is_contiguous()
+        if delta.dim() == 3:
+            assert delta.dtype == torch.float32 and delta.shape[1:] == residual.shape
+            parts, part_stride = delta.shape[0], residual.numel()
+        else:
+            assert delta.dtype == out.dtype and delta.shape == residual.shape
     if rows is None:
         assert residual.shape[0] == n
     else:
         assert rows.dtype == torch.int32 and rows.numel() == n
         write_residual = False
     wp, wf = _param(weight)
-    _check(library().pae_add_rmsnorm(code_of(out.dtype), residual.data_ptr(), _ptr(delta), wp, wf, float(eps),
+    _check(library().pae_add_rmsnorm(code_of(out.dtype), residual.data_ptr(), _ptr(delta), parts, part_stride,
+                                     wp, wf, float(eps),
                                      _ptr(rows), out.data_ptr(), n, H, 1 if write_residual else 0, _stream()))
 
 
@@ -181,12 +191,54 @@ def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, inv_f
                                        _stream()))
 
 
-def swiglu(out: torch.Tensor, x: torch.Tensor) -> None:
-    """out[t, j] = silu(x[t, j]) * x[t, I + j] for x of width 2 I."""
+def swiglu(out: torch.Tensor, x: torch.Tensor, block: int = 0) -> None:
+    """out[t, j] = silu(gate_j) * up_j for x of width 2 I: gate = x[:, :I], up = x[:, I:], or,
+    with `block` > 0, blocks of `block` gate features each followed by their up features."""
     _gpu(out, x)
     T, I = out.shape
     assert x.shape == (T, 2 * I) and x.dtype == out.dtype and x.is_contiguous() and out.is_contiguous()
-    _check(library().pae_swiglu(code_of(x.dtype), out.data_ptr(), x.data_ptr(), T, I, _stream()))
+    _check(library().pae_swiglu(code_of(x.dtype), out.data_ptr(), x.data_ptr(), T, I, block, _stream()))
+
+
+SKINNY_MAX_ROWS = 64
+EPI_BF16, EPI_F32, EPI_SWIGLU = 0, 1, 2
+
+
+def skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """The weight-streaming product takes bfloat16, at most 64 rows and rows of 16-byte multiples."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[0] <= SKINNY_MAX_ROWS
+            and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0 and a.stride(1) == 1)
+
+
+def skinny_splits(N: int, K: int) -> int:
+    """k ranges for a product whose consumer adds float32 partials: enough workgroups to fill the chip."""
+    tiles = -(-N // 16)
+    wanted = max(1, min(512 // tiles, K // 256, 8))
+    k_per = -(-(-(-K // wanted)) // 128) * 128
+    return -(-K // k_per)
+
+
+def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                epilogue: int = EPI_BF16, splits: int = 1) -> None:
+    """out = a @ w^T for at most 64 rows of `a`, reading `w` once.
+
+    EPI_BF16: out [M, N] bfloat16 (+bias).  EPI_F32: out [M, N] float32, or [splits, M, N]
+    partial sums over k ranges.  EPI_SWIGLU: w holds blocks of 16 gate rows followed by their 16
+    up rows; out [M, N / 2] = silu(gate) * up."""
+    _gpu(out, a, w, bias)
+    M, K_ = a.shape
+    N = w.shape[0]
+    assert skinny_supported(a, w) and w.shape == (N, K_) and w.is_contiguous() and out.is_contiguous()
+    if epilogue == EPI_SWIGLU:
+        assert out.shape == (M, N // 2) and out.dtype == torch.bfloat16 and splits == 1 and bias is None
+    elif epilogue == EPI_F32:
+        assert out.dtype == torch.float32
+        assert tuple(out.shape) == ((M, N) if splits == 1 and out.dim() == 2 else (splits, M, N))
+    else:
+        assert out.shape == (M, N) and out.dtype == torch.bfloat16 and splits == 1
+    bp, bf = _param(bias)
+    _check(library().pae_gemm_skinny(epilogue, out.data_ptr(), out.stride(-2), a.data_ptr(), a.stride(0),
+                                     w.data_ptr(), bp, bf, M, N, K_, splits, M * N, _stream()))
 
 
 def gemm_plain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:

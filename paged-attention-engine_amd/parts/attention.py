@@ -86,4 +86,4 @@ class PagedAttention(Part):
                 K.attn_prefill(attn, qkv, k_cache, v_cache, ctx.prefill_tiles, ctx.positions, table, *geometry)
         else:
             K.paged_attention_generic(attn, qkv, k_cache, v_cache, ctx.positions, ctx.tok_seq, table, *geometry)
-        return self.out(attn)
+        return self.out.branch(attn)

@@ -1,10 +1,15 @@
 """y = x W^T + b, the matrix product every part shares.
 
 The reference calls F.linear on weights stored (out_features, in_features)
-(engine/model.py:303-305,315,318-320).  In float32 this engine runs its own
-product kernel, which accumulates in float32 in k order with no reduced
-precision; in bfloat16 large products go to the platform's matrix library (as
-the reference's go to its library) and accumulate in float32.
+(engine/model.py:303-305,315,318-320).  Here:
+
+  float32    this engine's own product kernel: float32 fused multiply-adds in k
+             order, no reduced-precision matrix mode, each row independent of the
+             batch;
+  bfloat16   up to 64 rows (decode steps, small portions): the weight-streaming
+             matrix-core kernel, which reads W once; more rows: the platform's
+             matrix library, as the reference's products go to its library.
+             Both accumulate in float32.
 """
 
 from __future__ import annotations
@@ -23,19 +28,51 @@ class Linear:
         self.bias = bias
         self.out_features, self.in_features = weight.shape
 
-    def __call__(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-        out_dtype = out_dtype or x.dtype
-        out = torch.empty((x.shape[0], self.out_features), dtype=out_dtype, device=x.device)
-        if x.shape[0] == 0:
-            return out
-        if x.dtype == torch.float32 or out_dtype != x.dtype:
-            K.gemm_plain(out, x, self.weight, self.bias)
+    def _library(self, x: torch.Tensor) -> torch.Tensor:
+        out = torch.empty((x.shape[0], self.out_features), dtype=x.dtype, device=x.device)
+        bias = self.bias
+        if bias is None:
+            torch.mm(x, self.weight.t(), out=out)
         else:
-            bias = self.bias
-            if bias is not None and bias.dtype != x.dtype:
-                bias = bias.to(x.dtype)
-            if bias is None:
-                torch.mm(x, self.weight.t(), out=out)
-            else:
-                torch.addmm(bias, x, self.weight.t(), out=out)
+            torch.addmm(bias if bias.dtype == x.dtype else bias.to(x.dtype), x, self.weight.t(), out=out)
+        return out
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        """[M, N] in x's dtype."""
+        M = x.shape[0]
+        if x.dtype == torch.float32 or M == 0:
+            out = torch.empty((M, self.out_features), dtype=x.dtype, device=x.device)
+            if M:
+                K.gemm_plain(out, x, self.weight, self.bias)
+            return out
+        if K.skinny_supported(x, self.weight):
+            out = torch.empty((M, self.out_features), dtype=x.dtype, device=x.device)
+            K.gemm_skinny(out, x, self.weight, self.bias, K.EPI_BF16)
+            return out
+        return self._library(x)
+
+    def branch(self, x: torch.Tensor) -> torch.Tensor:
+        """The product as a residual branch's output: [M, N] in x's dtype, or float32
+        partial sums [P, M, N] that the next norm adds up in order (no bias then)."""
+        if x.dtype == torch.bfloat16 and self.bias is None and x.shape[0] and K.skinny_supported(x, self.weight):
+            splits = K.skinny_splits(self.out_features, self.in_features)
+            out = torch.empty((splits, x.shape[0], self.out_features), dtype=torch.float32, device=x.device)
+            K.gemm_skinny(out, x, self.weight, None, K.EPI_F32, splits)
+            return out
+        return self(x)
+
+    def float32(self, x: torch.Tensor) -> torch.Tensor:
+        """[M, N] float32 whatever x's dtype (the head's logits)."""
+        M = x.shape[0]
+        out = torch.empty((M, self.out_features), dtype=torch.float32, device=x.device)
+        if M == 0:
+            return out
+        if x.dtype == torch.float32:
+            K.gemm_plain(out, x, self.weight, self.bias)
+        elif x.shape[1] % 8 == 0:
+            for first in range(0, M, K.SKINNY_MAX_ROWS):
+                rows = slice(first, min(M, first + K.SKINNY_MAX_ROWS))
+                K.gemm_skinny(out[rows], x[rows], self.weight, self.bias, K.EPI_F32)
+        else:
+            K.gemm_plain(out, x, self.weight, self.bias)
         return out

@@ -24,13 +24,25 @@ class SwiGLU(Part):
                 prefix + "up_proj.weight": (s.intermediate_size, s.hidden_size),
                 prefix + "down_proj.weight": (s.hidden_size, s.intermediate_size)}
 
+    BLOCK = 16  # gate and up rows alternate in blocks of this many (the skinny product's gated epilogue)
+
     def bind(self, prefix, weights):
-        gate_up = torch.cat([weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]], dim=0)
+        gate, up = weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]
+        inter, hidden = gate.shape
+        self.block = self.BLOCK if (self.dtype == torch.bfloat16 and inter % self.BLOCK == 0) else 0
+        if self.block:
+            b = self.block
+            gate_up = torch.stack([gate.view(inter // b, b, hidden), up.view(inter // b, b, hidden)], dim=1)
+            gate_up = gate_up.reshape(2 * inter, hidden)
+        else:
+            gate_up = torch.cat([gate, up], dim=0)
         self.gate_up = Linear(self.matrix(gate_up))
         self.down = Linear(self.matrix(weights[prefix + "down_proj.weight"]))
 
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
-        both = self.gate_up(x)
         act = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
-        K.swiglu(act, both)
-        return self.down(act)
+        if self.block and x.shape[0] and K.skinny_supported(x, self.gate_up.weight):
+            K.gemm_skinny(act, x, self.gate_up.weight, None, K.EPI_SWIGLU)
+        else:
+            K.swiglu(act, self.gate_up(x), self.block)
+        return self.down.branch(act)

@@ -86,6 +86,75 @@ def test_gemm_plain(dtype, M, N, K_):
         assert torch.equal(one[0], out[M - 1])
 
 
+@pytest.mark.parametrize("M", [1, 8, 17, 64])
+@pytest.mark.parametrize("N,K_", [(2048, 1536), (1536, 8960), (50, 72), (777, 64), (96, 200)])
+def test_gemm_skinny(M, N, K_):
+    torch.manual_seed(M + N)
+    a = (torch.randn(M, K_) * 0.5).to(torch.bfloat16)
+    w = (torch.randn(N, K_) * 0.1).to(torch.bfloat16)
+    b = torch.randn(N).to(torch.bfloat16)
+    want = a.double() @ w.double().t()
+    scale = float(want.abs().max())
+    # bfloat16 out with bias
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    K().gemm_skinny(out, a.to(DEV), w.to(DEV), b.to(DEV), K().EPI_BF16)
+    assert (out.double().cpu() - (want + b.double())).abs().max() <= 2.0 ** -7 * (scale + 3)
+    # float32 out: one range, and partial sums over several k ranges added in order
+    out32 = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    K().gemm_skinny(out32, a.to(DEV), w.to(DEV), None, K().EPI_F32)
+    assert (out32.double().cpu() - want).abs().max() <= 2e-5 * scale
+    splits = K().skinny_splits(N, K_)
+    parts = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device=DEV)
+    K().gemm_skinny(parts, a.to(DEV), w.to(DEV), None, K().EPI_F32, splits)
+    assert (parts.sum(0).double().cpu() - want).abs().max() <= 2e-5 * scale
+    if K_ >= 1536:
+        assert splits > 1
+    # a row's result does not depend on the other rows
+    if M > 1:
+        one = torch.empty(1, N, dtype=torch.float32, device=DEV)
+        K().gemm_skinny(one, a[M - 1:].to(DEV), w.to(DEV), None, K().EPI_F32)
+        assert torch.equal(one[0], out32[M - 1])
+
+
+@pytest.mark.parametrize("M", [1, 8, 33])
+@pytest.mark.parametrize("inter,K_", [(8960, 1536), (176, 64), (48, 72)])
+def test_gemm_skinny_gated(M, inter, K_):
+    torch.manual_seed(inter)
+    a = torch.randn(M, K_).to(torch.bfloat16)
+    gate = (torch.randn(inter, K_) * 0.2).to(torch.bfloat16)
+    up = (torch.randn(inter, K_) * 0.2).to(torch.bfloat16)
+    want = plain.silu(a.double() @ gate.double().t()) * (a.double() @ up.double().t())
+    w = torch.stack([gate.view(inter // 16, 16, K_), up.view(inter // 16, 16, K_)], dim=1).reshape(2 * inter, K_)
+    out = torch.empty(M, inter, dtype=torch.bfloat16, device=DEV)
+    K().gemm_skinny(out, a.to(DEV), w.contiguous().to(DEV), None, K().EPI_SWIGLU)
+    assert (out.double().cpu() - want).abs().max() <= 2.0 ** -7 * float(want.abs().max())
+    # the separate gate kernel reads the same interleaved layout
+    both = (a.double() @ w.double().t()).to(torch.bfloat16)
+    out2 = torch.empty(M, inter, dtype=torch.bfloat16, device=DEV)
+    K().swiglu(out2, both.to(DEV), 16)
+    assert (out2.double().cpu() - want).abs().max() <= 2.0 ** -6 * float(want.abs().max())
+
+
+def test_add_rmsnorm_sums_float32_partials_in_order():
+    torch.manual_seed(4)
+    n, hidden, eps = 5, 200, 1e-6
+    res = torch.randn(n, hidden)
+    parts = torch.randn(3, n, hidden)
+    w = (1 + 0.1 * torch.randn(hidden)).to(torch.bfloat16)
+    summed = res + ((parts[0] + parts[1]) + parts[2])
+    normed = (summed * torch.rsqrt(summed.pow(2).mean(-1, keepdim=True) + eps)).to(torch.bfloat16)
+    want = (w.float() * normed.float()).to(torch.bfloat16).float()
+    r = res.to(DEV)
+    out = torch.empty(n, hidden, dtype=torch.bfloat16, device=DEV)
+    K().add_rmsnorm(r, parts.to(DEV), w.to(DEV), eps, out)
+    assert torch.allclose(r.cpu(), summed, atol=1e-6)
+    assert (out.float().cpu() - want).abs().max() <= 2.0 ** -7 * float(want.abs().max())
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, hidden, dtype=torch.bfloat16, device=DEV)
+    K().add_rmsnorm(res.to(DEV), parts.to(DEV), w.to(DEV), eps, out2, rows)
+    assert (out2.float().cpu() - want[[4, 1]]).abs().max() <= 2.0 ** -7 * float(want.abs().max())
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_swiglu(dtype):
     x = (torch.randn(9, 2 * 177) * 3).to(DT[dtype])
