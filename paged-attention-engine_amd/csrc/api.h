@@ -29,15 +29,16 @@ int pae_paged_attention_generic(int dtype, void* out, int64_t out_stride, const 
                                 const int* tok_seq, const int* block_tables, int max_blocks, int bs,
                                 int num_tokens, int nh, int nkv, int hd, float scale, int window,
                                 hipStream_t stream);
+int pae_attn_decode_split();
 int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
                          const void* v_cache, const int* dec_tok, int num_dec, const int* positions,
                          const int* tok_seq, const int* block_tables, int max_blocks, int bs, int nh, int nkv,
-                         int hd, float scale, int window, int split_len, void* part_acc, void* part_ml,
-                         hipStream_t stream);
+                         int hd, float scale, int window, void* part_acc, void* part_ml, hipStream_t stream);
 int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
                           const void* v_cache, const int* tiles, int num_tiles, const int* positions,
                           const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,
                           int window, hipStream_t stream);
+int pae_sample_chunks(int vocab);
 int pae_sample(int* tokens, const float* logits, int64_t ld, const float* temperature, const float* uniform,
-               int num_rows, int vocab, hipStream_t stream);
+               int num_rows, int vocab, float* chunk_max, int* chunk_arg, double* chunk_sum, hipStream_t stream);
 }

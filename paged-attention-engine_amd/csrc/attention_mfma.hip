@@ -14,8 +14,8 @@
 // decode:  one workgroup per (sequence with a single new token, kv head, split of
 //          the keys); the columns are the query heads that share the kv head, so a
 //          page is read once for all of them.  Four wavefronts take pages in turn
-//          and merge in LDS; splits are merged by a second kernel.  Splits start at
-//          multiples of the split length from position 0.
+//          and merge in LDS; the last workgroup to finish merges the splits.  Splits
+//          start at multiples of the split length from position 0.
 // prefill: one wavefront per (32 consecutive tokens of a sequence, query head).
 //
 // Masking is the reference's rule (engine/attention.py:474-487: key j visible iff
@@ -100,21 +100,31 @@ __device__ __forceinline__ void load_kv_tile(bf16x8 (&kf)[HD / 32], s16x4 (&vf)[
 }
 
 // ------------------------------------------------------------------ decode
-// part_acc[(token, head, split)][hd] unnormalised, part_ml[(token, head, split)][2] = (max, sum)
-template <int HD>
+// Split s of a token covers keys [s * 64 TPW, (s + 1) * 64 TPW); wavefront w of its
+// workgroup takes the 16-key tiles w, w + 4, ... of the split, all loaded before the
+// first is used.  Each workgroup leaves its partial result (unnormalised sums, running
+// maximum and sum of weights per head) in `part_*`; a second kernel adds the partials
+// in split order.  (Merging in the last workgroup to finish, found by a ticket
+// counter, was tried: the device-wide fences it needs write back and invalidate L2
+// for every workgroup and cost more than the second launch.)
+//   part_acc[((token * nkv + kvh) * max_splits + split) * g + head in group][HD]
+//   part_ml [ ... same index ... ][2] = (maximum in log2 units, sum)
+template <int HD, int TPW>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
-    float* __restrict__ part_acc, float* __restrict__ part_ml, int max_splits, const bf16_t* __restrict__ q,
-    int64_t q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
-    const int* __restrict__ dec_tok, const int* __restrict__ positions, const int* __restrict__ tok_seq,
-    const int* __restrict__ block_tables, int max_blocks, int bs, int nh, int nkv, float scale_log2,
-    int window, int split_len) {
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int max_splits,
+    const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ dec_tok,
+    const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_tables,
+    int max_blocks, int bs, int nh, int nkv, float scale_log2, int window) {
+  constexpr int SPLIT = 64 * TPW;
   const int split = blockIdx.x, kvh = blockIdx.y;
   const int tok = dec_tok[blockIdx.z];
   const int pos[1] = {positions[tok]};
   const int start[1] = {(window > 0 && pos[0] - window + 1 > 0) ? pos[0] - window + 1 : 0};
-  const int lo = max(split * split_len, start[0] / 16 * 16);
-  const int hi = min((split + 1) * split_len, pos[0] + 1);  // keys [lo, hi)
-  if (lo >= hi) return;
+  const int s_first = start[0] / SPLIT, s_last = pos[0] / SPLIT;
+  if (split < s_first || split > s_last) return;
+  const int lo = max(split * SPLIT, start[0] / 16 * 16);
+  const int hi = min((split + 1) * SPLIT, pos[0] + 1);  // keys [lo, hi), not empty
   const int* table = block_tables + (int64_t)tok_seq[tok] * max_blocks;
   const int g = nh / nkv;
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
@@ -138,83 +148,97 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   for (int t = 0; t < HD / 16; ++t) st.acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   const int page_elems = bs * HD;
-  // 16-key tiles of the split, taken by the four wavefronts in turn
   const int tile_lo = lo / 16, tile_hi = (hi + 15) / 16;
-  bf16x8 kf[HD / 32];
-  s16x4 vf[HD / 16];
-  for (int tile = tile_lo + wave; tile < tile_hi; tile += 4) {
-    const int key0 = tile * 16;
-    const int blk = table[key0 / bs];
-    const int64_t base = ((int64_t)blk * nkv + kvh) * page_elems;
-    load_kv_tile<HD>(kf, vf, k_cache + base + (int64_t)(key0 % bs) * HD, v_cache + base + key0 % bs, bs);
-    attn_tile<HD, 1>(st, kf, vf, qf, key0, pos, start, scale_log2);
+  bf16x8 kf[TPW][HD / 32];
+  s16x4 vf[TPW][HD / 16];
+#pragma unroll
+  for (int j = 0; j < TPW; ++j) {  // a tile past the end is loaded from the first tile's place and not used
+    const int tile = tile_lo + wave + 4 * j;
+    const int key0 = (tile < tile_hi ? tile : tile_lo) * 16;
+    const int64_t base = ((int64_t)table[key0 / bs] * nkv + kvh) * page_elems;
+    load_kv_tile<HD>(kf[j], vf[j], k_cache + base + (int64_t)(key0 % bs) * HD, v_cache + base + key0 % bs, bs);
+  }
+#pragma unroll
+  for (int j = 0; j < TPW; ++j) {
+    const int tile = tile_lo + wave + 4 * j;
+    if (tile < tile_hi) attn_tile<HD, 1>(st, kf[j], vf[j], qf, tile * 16, pos, start, scale_log2);
   }
 
-  // merge wavefronts 1..3 into wavefront 0, one after the other: every lane of a
-  // wavefront holds the same (column, features) as the same lane of wavefront 0
-  extern __shared__ float s_buf[];  // [HD / 4 + 2][64]
-  for (int w = 1; w < 4; ++w) {
-    if (wave == w) {
+  // wavefronts 1..3 hand their state to wavefront 0 through LDS; every lane of a wavefront
+  // holds the same (column, features) as the same lane of wavefront 0
+  extern __shared__ float s_buf[];  // [3][HD / 4 + 2][64]
+  constexpr int ROWS = HD / 4 + 2;
+  if (wave > 0) {
+    float* mine = s_buf + (wave - 1) * ROWS * PAE_WAVE;
 #pragma unroll
-      for (int t = 0; t < HD / 16; ++t)
+    for (int t = 0; t < HD / 16; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) s_buf[(4 * t + i) * PAE_WAVE + lane] = st.acc[0][t][i];
-      s_buf[(HD / 4) * PAE_WAVE + lane] = st.m[0];
-      s_buf[(HD / 4 + 1) * PAE_WAVE + lane] = st.l[0];
-    }
-    __syncthreads();
-    if (wave == 0) {
-      const float mw = s_buf[(HD / 4) * PAE_WAVE + lane];
+      for (int i = 0; i < 4; ++i) mine[(4 * t + i) * PAE_WAVE + lane] = st.acc[0][t][i];
+    mine[(HD / 4) * PAE_WAVE + lane] = st.m[0];
+    mine[(HD / 4 + 1) * PAE_WAVE + lane] = st.l[0];
+  }
+  __syncthreads();
+  const int64_t group_slot = ((int64_t)blockIdx.z * nkv + kvh) * max_splits;
+  if (wave == 0) {
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+      const float* theirs = s_buf + w * ROWS * PAE_WAVE;
+      const float mw = theirs[(HD / 4) * PAE_WAVE + lane];
       const float m_new = fmaxf(st.m[0], mw);
       const float f0 = exp2f(st.m[0] - m_new), fw = exp2f(mw - m_new);
 #pragma unroll
       for (int t = 0; t < HD / 16; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          st.acc[0][t][i] = st.acc[0][t][i] * f0 + s_buf[(4 * t + i) * PAE_WAVE + lane] * fw;
-      st.l[0] = st.l[0] * f0 + s_buf[(HD / 4 + 1) * PAE_WAVE + lane] * fw;
+        for (int i = 0; i < 4; ++i) st.acc[0][t][i] = st.acc[0][t][i] * f0 + theirs[(4 * t + i) * PAE_WAVE + lane] * fw;
+      st.l[0] = st.l[0] * f0 + theirs[(HD / 4 + 1) * PAE_WAVE + lane] * fw;
       st.m[0] = m_new;
     }
-    __syncthreads();
-  }
-  if (wave != 0) return;
-  float l = st.l[0];
-  l += __shfl_xor(l, 16, PAE_WAVE);
-  l += __shfl_xor(l, 32, PAE_WAVE);
-  if (col < g) {
-    const int64_t slot = ((int64_t)blockIdx.z * nh + kvh * g + col) * max_splits + split;
+    float l = st.l[0];
+    l += __shfl_xor(l, 16, PAE_WAVE);
+    l += __shfl_xor(l, 32, PAE_WAVE);
+    if (col < g) {
+      const int64_t slot = (group_slot + split) * g + col;
 #pragma unroll
-    for (int t = 0; t < HD / 16; ++t)
-      *reinterpret_cast<f32x4*>(part_acc + slot * HD + 16 * t + 4 * g4) = st.acc[0][t];
-    if (g4 == 0) {
-      part_ml[slot * 2] = st.m[0];
-      part_ml[slot * 2 + 1] = l;
+      for (int t = 0; t < HD / 16; ++t)
+        *reinterpret_cast<f32x4*>(part_acc + slot * HD + 16 * t + 4 * g4) = st.acc[0][t];
+      if (g4 == 0) {
+        part_ml[slot * 2] = st.m[0];
+        part_ml[slot * 2 + 1] = l;
+      }
     }
   }
 }
 
-// out[token, head, :] = sum over the splits that hold keys, in split order
-template <int HD>
-__global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
-                                         const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                                         int max_splits, const int* __restrict__ dec_tok,
-                                         const int* __restrict__ positions, int nh, int window, int split_len) {
-  const int head = blockIdx.x;
+// Adds a token's partials in split order and writes the output: one workgroup per
+// (token, kv head), launched after the kernel above.
+template <int HD, int TPW>
+__global__ __launch_bounds__(256) void attn_decode_merge_kernel(
+    bf16_t* __restrict__ out, int64_t out_stride, const float* __restrict__ part_acc,
+    const float* __restrict__ part_ml, int max_splits, const int* __restrict__ dec_tok,
+    const int* __restrict__ positions, int nh, int nkv, int window) {
+  constexpr int SPLIT = 64 * TPW;
+  const int kvh = blockIdx.x;
   const int tok = dec_tok[blockIdx.y];
   const int pos = positions[tok];
   const int start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int first = start / split_len, last = pos / split_len;
-  const int64_t slot0 = ((int64_t)blockIdx.y * nh + head) * max_splits;
-  float m = NEG_BIG;
-  for (int s = first; s <= last; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+  const int s_first = start / SPLIT, nsplits = pos / SPLIT - s_first + 1;
+  const int g = nh / nkv;
+  const int64_t group_slot = ((int64_t)blockIdx.y * nkv + kvh) * max_splits;
+  for (int idx = threadIdx.x; idx < g * HD; idx += blockDim.x) {
+    const int c = idx / HD, d = idx % HD;
+    const int64_t slot0 = (group_slot + s_first) * g + c;  // consecutive splits are g slots apart
+    float m = NEG_BIG;
+#pragma unroll 8
+    for (int sp = 0; sp < nsplits; ++sp) m = fmaxf(m, part_ml[(slot0 + (int64_t)sp * g) * 2]);
     float a = 0.f, l = 0.f;
-    for (int s = first; s <= last; ++s) {
-      const float f = exp2f(part_ml[(slot0 + s) * 2] - m);
-      a += f * part_acc[(slot0 + s) * HD + d];
-      l += f * part_ml[(slot0 + s) * 2 + 1];
+#pragma unroll 8
+    for (int sp = 0; sp < nsplits; ++sp) {
+      const int64_t slot = slot0 + (int64_t)sp * g;
+      const float f = exp2f(part_ml[slot * 2] - m);
+      a += f * part_acc[slot * HD + d];
+      l += f * part_ml[slot * 2 + 1];
     }
-    out[(int64_t)tok * out_stride + (int64_t)head * HD + d] = __float2bfloat16(a / l);
+    out[(int64_t)tok * out_stride + (int64_t)(kvh * g + c) * HD + d] = __float2bfloat16(a / l);
   }
 }
 
@@ -313,27 +337,32 @@ static int check_common(const char* what, int nh, int nkv, int hd, int bs, int m
   return 0;
 }
 
-// Workspace: part_acc holds num_dec * nh * max_splits * hd floats, part_ml num_dec * nh * max_splits * 2.
+// Keys per split of the decode kernel (fixed, so a token's result does not depend on the batch).
+#define DECODE_TPW 2
+extern "C" int pae_attn_decode_split() { return 64 * DECODE_TPW; }
+
+// Workspace: part_acc holds num_dec * nh * max_splits * hd floats, part_ml num_dec * nh * max_splits * 2,
+// max_splits = ceil(max_blocks * bs / pae_attn_decode_split()).
 extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                     const void* k_cache, const void* v_cache, const int* dec_tok, int num_dec,
                                     const int* positions, const int* tok_seq, const int* block_tables,
                                     int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
-                                    int split_len, void* part_acc, void* part_ml, hipStream_t stream) {
+                                    void* part_acc, void* part_ml, hipStream_t stream) {
   if (int rc = check_common("attn_decode", nh, nkv, hd, bs, max_blocks, window)) return rc;
-  PAE_REQUIRE(split_len >= 64 && split_len % 64 == 0, "attn_decode: split length %d is not a multiple of 64", split_len);
   PAE_REQUIRE(num_dec <= 65535 && nkv <= 65535, "attn_decode: grid too large");
   if (num_dec <= 0) return 0;
+  const int split_len = 64 * DECODE_TPW;
   const int max_splits = (int)(((int64_t)max_blocks * bs + split_len - 1) / split_len);
   const float scale_log2 = scale * LOG2E;
-  dim3 grid(max_splits, nkv, num_dec), merge_grid(nh, num_dec);
-#define CALL(HD)                                                                                              \
-  attn_decode_kernel<HD><<<grid, 256, (size_t)(HD / 4 + 2) * PAE_WAVE * sizeof(float), stream>>>(                         \
-      (float*)part_acc, (float*)part_ml, max_splits, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,      \
+  dim3 grid(max_splits, nkv, num_dec), merge_grid(nkv, num_dec);
+#define CALL(HD)                                                                                            \
+  attn_decode_kernel<HD, DECODE_TPW><<<grid, 256, (size_t)3 * (HD / 4 + 2) * PAE_WAVE * sizeof(float), stream>>>( \
+      (float*)part_acc, (float*)part_ml, max_splits, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,     \
       (const bf16_t*)v_cache, dec_tok, positions, tok_seq, block_tables, max_blocks, bs, nh, nkv, scale_log2, \
-      window, split_len);                                                                                     \
-  attn_decode_merge_kernel<HD><<<merge_grid, 64, 0, stream>>>((bf16_t*)out, out_stride, (const float*)part_acc, \
-                                                              (const float*)part_ml, max_splits, dec_tok,     \
-                                                              positions, nh, window, split_len)
+      window);                                                                                               \
+  attn_decode_merge_kernel<HD, DECODE_TPW><<<merge_grid, 256, 0, stream>>>(                                  \
+      (bf16_t*)out, out_stride, (const float*)part_acc, (const float*)part_ml, max_splits, dec_tok, positions, \
+      nh, nkv, window)
   FOR_HEAD_DIM(hd, CALL)
 #undef CALL
   return pae_check_launch("attn_decode");

@@ -50,16 +50,77 @@ __device__ __forceinline__ float pending_at(const void* delta, int parts, int64_
   return sum;
 }
 
-template <typename T, int NT>
-__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const void* __restrict__ delta, int parts,
-                                   int64_t part_stride, const void* __restrict__ weight, int w_is_f32,
-                                   float eps, const int* __restrict__ rows, T* __restrict__ out, int hidden,
-                                   int write_residual) {
+#define RMS_MAXP 8
+// EPT > 0: each thread keeps its EPT elements of the row in registers (hidden <= NT * EPT):
+// all loads are issued before the first is used and the row is read once.
+// EPT == 0: any width, two passes over the row.
+template <typename T, int NT, int EPT>
+__global__ __launch_bounds__(NT) void add_rmsnorm_kernel(float* __restrict__ residual,
+                                                         const void* __restrict__ delta, int parts,
+                                                         int64_t part_stride, const void* __restrict__ weight,
+                                                         int w_is_f32, float eps, const int* __restrict__ rows,
+                                                         T* __restrict__ out, int hidden, int write_residual) {
   __shared__ float scratch[NT / PAE_WAVE];
   const int b = blockIdx.x;
   const int64_t src = rows ? rows[b] : b;
   float* res = residual + src * hidden;
   T* dst = out + (int64_t)b * hidden;
+  if (EPT > 0) {
+    float r[EPT > 0 ? EPT : 1];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int i = threadIdx.x + e * NT;
+      r[e] = i < hidden ? res[i] : 0.f;
+    }
+    if (delta) {
+      if (parts == 0) {
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) {
+          const int i = threadIdx.x + e * NT;
+          if (i < hidden) r[e] += to_f32(((const T*)delta)[src * hidden + i]);
+        }
+      } else {
+        // partial sums are added in order; the first RMS_MAXP of them are loaded without
+        // branches (from a clamped address, dropped by a select) so that all are in flight at once
+        float psum[EPT > 0 ? EPT : 1];
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) psum[e] = 0.f;
+#pragma unroll
+        for (int p = 0; p < RMS_MAXP; ++p) {
+          const float* part = (const float*)delta + (int64_t)(p < parts ? p : parts - 1) * part_stride + src * hidden;
+#pragma unroll
+          for (int e = 0; e < EPT; ++e) {
+            const int i = threadIdx.x + e * NT;
+            const float v = part[i < hidden ? i : 0];
+            psum[e] += (p < parts && i < hidden) ? v : 0.f;
+          }
+        }
+        for (int p = RMS_MAXP; p < parts; ++p)
+#pragma unroll
+          for (int e = 0; e < EPT; ++e) {
+            const int i = threadIdx.x + e * NT;
+            if (i < hidden) psum[e] += ((const float*)delta)[p * part_stride + src * hidden + i];
+          }
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) r[e] += psum[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int i = threadIdx.x + e * NT;
+      if (write_residual && delta && i < hidden) res[i] = r[e];
+      ss += r[e] * r[e];
+    }
+    const float total = block_sum<NT / PAE_WAVE>(ss, scratch);
+    const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int i = threadIdx.x + e * NT;
+      if (i < hidden) dst[i] = from_f32<T>(load_param(weight, w_is_f32, i) * round_to<T>(r[e] * inv));
+    }
+    return;
+  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += NT) {
     float r = res[i];
@@ -84,14 +145,24 @@ extern "C" int pae_add_rmsnorm(int dtype, void* residual, const void* delta, int
   PAE_REQUIRE(num_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d H=%d", num_rows, hidden);
   PAE_REQUIRE(!(rows && write_residual), "add_rmsnorm: a row gather may not write the residual back");
   if (num_rows == 0) return 0;
-  if (dtype == PAE_F32)
-    add_rmsnorm_kernel<float, 256><<<num_rows, 256, 0, stream>>>(
-        (float*)residual, delta, parts, part_stride, weight, w_is_f32, eps, rows, (float*)out, hidden, write_residual);
-  else if (dtype == PAE_BF16)
-    add_rmsnorm_kernel<bf16_t, 256><<<num_rows, 256, 0, stream>>>(
-        (float*)residual, delta, parts, part_stride, weight, w_is_f32, eps, rows, (bf16_t*)out, hidden, write_residual);
-  else
+#define RMS_LAUNCH(T, EPT)                                                                                  \
+  add_rmsnorm_kernel<T, 256, EPT><<<num_rows, 256, 0, stream>>>((float*)residual, delta, parts, part_stride, \
+                                                                weight, w_is_f32, eps, rows, (T*)out, hidden, \
+                                                                write_residual)
+#define RMS_BY_WIDTH(T)                          \
+  if (hidden <= 256 * 2) RMS_LAUNCH(T, 2);       \
+  else if (hidden <= 256 * 8) RMS_LAUNCH(T, 8);  \
+  else if (hidden <= 256 * 32) RMS_LAUNCH(T, 32); \
+  else RMS_LAUNCH(T, 0)
+  if (dtype == PAE_F32) {
+    RMS_BY_WIDTH(float);
+  } else if (dtype == PAE_BF16) {
+    RMS_BY_WIDTH(bf16_t);
+  } else {
     return pae_fail("add_rmsnorm: unknown dtype code %d", dtype);
+  }
+#undef RMS_BY_WIDTH
+#undef RMS_LAUNCH
   return pae_check_launch("add_rmsnorm");
 }
 

@@ -1,97 +1,191 @@
 // Picking tokens from float32 logits: argmax (first maximum wins, as torch.argmax
 // does in the reference, engine/scheduler.py:610) and inverse-CDF sampling from
 // softmax(logits / temperature) with a uniform number per row that the host
-// derives from (seed, request, token index).  One block per row; every sum runs
-// in a fixed order over the vocabulary, so a row's token does not depend on the
-// other rows of the batch.
+// derives from (seed, request, token index).
+//
+// A row is cut into `chunks` contiguous chunks so that the vocabulary is read by
+// many workgroups at once:
+//   1. every chunk finds its maximum (and where it first occurs);
+//   2. (only if a row samples) every chunk sums exp((x - row max) / T) in double,
+//      thread by thread over contiguous segments and then segment by segment, so
+//      that the sums follow index order;
+//   3. one workgroup per row picks the first maximum, or finds the chunk, the
+//      segment and the index at which the cumulative sum first exceeds u * total,
+//      repeating step 2's additions exactly.
+// Every sum runs in a fixed order, so a row's token does not depend on the batch.
 #include "common.h"
 #include "api.h"
 
 #define SAMPLE_NT 256
 
-// tokens[r] = temperature[r] == 0 ? argmax : first index whose cumulative
-// probability exceeds u[r] * total.
-__global__ __launch_bounds__(SAMPLE_NT) void sample_kernel(int* __restrict__ tokens,
-                                                           const float* __restrict__ logits, int64_t ld,
-                                                           const float* __restrict__ temperature,
-                                                           const float* __restrict__ uniform, int vocab) {
-  __shared__ float s_max[SAMPLE_NT];
-  __shared__ int s_idx[SAMPLE_NT];
-  __shared__ double s_sum[SAMPLE_NT];
-  __shared__ double s_target;
-  __shared__ int s_segment;
-  const int r = blockIdx.x;
-  const int tid = threadIdx.x;
-  const float* row = logits + (int64_t)r * ld;
-  // a contiguous segment of the vocabulary per thread, so prefix sums follow index order
-  const int per = (vocab + SAMPLE_NT - 1) / SAMPLE_NT;
-  const int lo = tid * per < vocab ? tid * per : vocab;
-  const int hi = lo + per < vocab ? lo + per : vocab;
+__device__ __forceinline__ void chunk_bounds(int vocab, int chunks, int c, int& lo, int& hi, int& per) {
+  const int size = (vocab + chunks - 1) / chunks;
+  lo = min(c * size, vocab);
+  hi = min(lo + size, vocab);
+  per = (size + SAMPLE_NT - 1) / SAMPLE_NT;  // elements of a thread's contiguous segment
+}
 
+__global__ __launch_bounds__(SAMPLE_NT) void sample_chunk_max_kernel(float* __restrict__ chunk_max,
+                                                                     int* __restrict__ chunk_arg,
+                                                                     const float* __restrict__ logits, int64_t ld,
+                                                                     int vocab, int chunks) {
+  __shared__ float s_val[SAMPLE_NT];
+  __shared__ int s_idx[SAMPLE_NT];
+  const int c = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+  int lo, hi, per;
+  chunk_bounds(vocab, chunks, c, lo, hi, per);
+  const float* row = logits + (int64_t)r * ld;
   float best = -INFINITY;
   int best_i = -1;
-  for (int i = lo; i < hi; ++i) {
+  for (int i = lo + tid; i < hi; i += SAMPLE_NT) {  // ascending per thread: strict > keeps the first
     const float x = row[i];
     if (best_i < 0 || x > best) { best = x; best_i = i; }
   }
-  s_max[tid] = best;
+  s_val[tid] = best;
   s_idx[tid] = best_i;
   __syncthreads();
-  if (tid == 0) {  // segments in index order, strict comparison: the first maximum wins
-    float b = s_max[0];
-    int bi = s_idx[0];
-    for (int w = 1; w < SAMPLE_NT; ++w)
-      if (s_idx[w] >= 0 && s_max[w] > b) { b = s_max[w]; bi = s_idx[w]; }
-    s_max[0] = b;
-    s_idx[0] = bi;
+  for (int step = SAMPLE_NT / 2; step > 0; step >>= 1) {
+    if (tid < step) {
+      const float ov = s_val[tid + step];
+      const int oi = s_idx[tid + step];
+      const int mi = s_idx[tid];
+      if (oi >= 0 && (mi < 0 || ov > s_val[tid] || (ov == s_val[tid] && oi < mi))) { s_val[tid] = ov; s_idx[tid] = oi; }
+    }
+    __syncthreads();
   }
-  __syncthreads();
-  const float row_max = s_max[0];
-  const int arg = s_idx[0];
-  const float temp = temperature ? temperature[r] : 0.f;
-  if (!(temp > 0.f)) {
-    if (tid == 0) tokens[r] = arg;
-    return;
+  if (tid == 0) {
+    chunk_max[r * chunks + c] = s_val[0];
+    chunk_arg[r * chunks + c] = s_idx[0];
   }
-  const float inv_t = 1.0f / temp;
-  double part = 0.0;
-  for (int i = lo; i < hi; ++i) part += (double)expf((row[i] - row_max) * inv_t);
-  s_sum[tid] = part;
+}
+
+// Sum of exp((x - row_max) * inv_t) over this thread's contiguous segment of the chunk.
+__device__ __forceinline__ double segment_sum(const float* row, int lo, int hi, int per, int tid, float row_max,
+                                              float inv_t) {
+  const int a = min(lo + tid * per, hi), b = min(a + per, hi);
+  double sum = 0.0;
+  for (int i = a; i < b; ++i) sum += (double)expf((row[i] - row_max) * inv_t);
+  return sum;
+}
+
+__device__ __forceinline__ float row_maximum(const float* chunk_max, int r, int chunks) {
+  float m = chunk_max[r * chunks];
+  for (int c = 1; c < chunks; ++c) m = fmaxf(m, chunk_max[r * chunks + c]);
+  return m;
+}
+
+__global__ __launch_bounds__(SAMPLE_NT) void sample_chunk_sum_kernel(double* __restrict__ chunk_sum,
+                                                                     const float* __restrict__ chunk_max,
+                                                                     const float* __restrict__ logits, int64_t ld,
+                                                                     const float* __restrict__ temperature,
+                                                                     int vocab, int chunks) {
+  __shared__ double s_seg[SAMPLE_NT];
+  const int c = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+  const float temp = temperature[r];
+  if (!(temp > 0.f)) return;
+  int lo, hi, per;
+  chunk_bounds(vocab, chunks, c, lo, hi, per);
+  const float* row = logits + (int64_t)r * ld;
+  s_seg[tid] = segment_sum(row, lo, hi, per, tid, row_maximum(chunk_max, r, chunks), 1.0f / temp);
   __syncthreads();
   if (tid == 0) {
     double total = 0.0;
-    for (int w = 0; w < SAMPLE_NT; ++w) total += s_sum[w];
+    for (int t = 0; t < SAMPLE_NT; ++t) total += s_seg[t];
+    chunk_sum[r * chunks + c] = total;
+  }
+}
+
+__global__ __launch_bounds__(SAMPLE_NT) void sample_pick_kernel(int* __restrict__ tokens,
+                                                                const float* __restrict__ chunk_max,
+                                                                const int* __restrict__ chunk_arg,
+                                                                const double* __restrict__ chunk_sum,
+                                                                const float* __restrict__ logits, int64_t ld,
+                                                                const float* __restrict__ temperature,
+                                                                const float* __restrict__ uniform, int vocab,
+                                                                int chunks) {
+  __shared__ double s_seg[SAMPLE_NT];
+  __shared__ double s_before;
+  __shared__ int s_where;
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const float temp = temperature ? temperature[r] : 0.f;
+  if (!(temp > 0.f)) {
+    if (tid == 0) {  // chunks in index order, strict comparison: the first maximum wins
+      float best = chunk_max[r * chunks];
+      int arg = chunk_arg[r * chunks];
+      for (int c = 1; c < chunks; ++c)
+        if (chunk_arg[r * chunks + c] >= 0 && (arg < 0 || chunk_max[r * chunks + c] > best)) {
+          best = chunk_max[r * chunks + c];
+          arg = chunk_arg[r * chunks + c];
+        }
+      tokens[r] = arg;
+    }
+    return;
+  }
+  const float* row = logits + (int64_t)r * ld;
+  const float row_max = row_maximum(chunk_max, r, chunks);
+  if (tid == 0) {
+    double total = 0.0;
+    for (int c = 0; c < chunks; ++c) total += chunk_sum[r * chunks + c];
     const double target = (double)uniform[r] * total;
     double run = 0.0;
-    int seg = -1;
-    for (int w = 0; w < SAMPLE_NT; ++w) {
-      const double v = s_sum[w];
-      s_sum[w] = run;  // exclusive prefix
-      if (seg < 0 && run + v > target) seg = w;
+    int where = -1;
+    for (int c = 0; c < chunks; ++c) {
+      const double v = chunk_sum[r * chunks + c];
+      if (run + v > target) { where = c; break; }
       run += v;
     }
-    s_target = target;
-    s_segment = seg;
-    if (seg < 0) tokens[r] = vocab - 1;  // u * total rounded up to the total
+    s_where = where;
+    s_before = target - run;  // what is left to cover inside the chunk
+    if (where < 0) tokens[r] = vocab - 1;  // u * total rounded up to the total
   }
   __syncthreads();
-  if (tid == s_segment) {
-    double run = s_sum[tid];
-    int pick = hi - 1;
-    for (int i = lo; i < hi; ++i) {
+  const int c = s_where;
+  if (c < 0) return;
+  int lo, hi, per;
+  chunk_bounds(vocab, chunks, c, lo, hi, per);
+  const float inv_t = 1.0f / temp;
+  s_seg[tid] = segment_sum(row, lo, hi, per, tid, row_max, inv_t);
+  __syncthreads();
+  if (tid == 0) {
+    const double target = s_before;
+    double run = 0.0;
+    int seg = SAMPLE_NT - 1;
+    for (int t = 0; t < SAMPLE_NT; ++t) {
+      if (run + s_seg[t] > target) { seg = t; break; }
+      run += s_seg[t];
+    }
+    const int a = min(lo + seg * per, hi), b = min(a + per, hi);
+    int pick = b - 1 >= a ? b - 1 : hi - 1;
+    for (int i = a; i < b; ++i) {
       run += (double)expf((row[i] - row_max) * inv_t);
-      if (run > s_target) { pick = i; break; }
+      if (run > target) { pick = i; break; }
     }
     tokens[r] = pick;
   }
 }
 
+extern "C" int pae_sample_chunks(int vocab) {
+  const int chunks = (vocab + 1023) / 1024;
+  return chunks < 1 ? 1 : (chunks > 128 ? 128 : chunks);
+}
+
+// Workspace: chunk_max and chunk_arg hold num_rows * pae_sample_chunks(vocab) values,
+// chunk_sum as many doubles (needed only with temperatures).
 extern "C" int pae_sample(int* tokens, const float* logits, int64_t ld, const float* temperature,
-                          const float* uniform, int num_rows, int vocab, hipStream_t stream) {
+                          const float* uniform, int num_rows, int vocab, float* chunk_max, int* chunk_arg,
+                          double* chunk_sum, hipStream_t stream) {
   PAE_REQUIRE(num_rows >= 0 && vocab > 0 && ld >= vocab, "sample: bad sizes rows=%d V=%d ld=%lld", num_rows,
               vocab, (long long)ld);
-  PAE_REQUIRE(!temperature || uniform, "sample: temperatures need uniform numbers");
+  PAE_REQUIRE(!temperature || (uniform && chunk_sum), "sample: temperatures need uniform numbers and sums");
+  PAE_REQUIRE(num_rows <= 65535, "sample: %d rows exceed the grid", num_rows);
   if (num_rows == 0) return 0;
-  sample_kernel<<<num_rows, SAMPLE_NT, 0, stream>>>(tokens, logits, ld, temperature, uniform, vocab);
+  const int chunks = pae_sample_chunks(vocab);
+  dim3 grid(chunks, num_rows);
+  sample_chunk_max_kernel<<<grid, SAMPLE_NT, 0, stream>>>(chunk_max, chunk_arg, logits, ld, vocab, chunks);
+  if (temperature)
+    sample_chunk_sum_kernel<<<grid, SAMPLE_NT, 0, stream>>>(chunk_sum, chunk_max, logits, ld, temperature, vocab,
+                                                            chunks);
+  sample_pick_kernel<<<num_rows, SAMPLE_NT, 0, stream>>>(tokens, chunk_max, chunk_arg, chunk_sum, logits, ld,
+                                                         temperature, uniform, vocab, chunks);
   return pae_check_launch("sample");
 }

@@ -74,6 +74,20 @@ class Model:
         else:
             self.head = Linear(weights[plan.head_name].to(device=self.device, dtype=self.dtype).contiguous())
 
+    @property
+    def graph_safe(self) -> bool:
+        """Can a step of this model be recorded as a HIP graph?  Every part must launch
+        device work only, and every matrix product must go through this engine's own
+        kernels (library products may record memory clears into a graph)."""
+        if not (all(block.graph_safe for block in self.blocks) and self.final_norm.graph_safe):
+            return False
+        if self.dtype == torch.float32:
+            return True
+        widths = [self.plan.hidden_size]
+        for block in self.blocks:
+            widths += getattr(block, "product_widths", lambda: [1])()
+        return all(w % 8 == 0 for w in widths)
+
     # ------------------------------------------------------------------ cache needs
     def cache_specs(self):
         """(paged, states): per schedule stop, what it keeps per token / per request."""

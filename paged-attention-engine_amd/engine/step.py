@@ -33,18 +33,40 @@ class StepEntry:
     want: Tuple[int, ...] = ()  # places among token_ids whose logits are returned
 
 
+class _CapturedStep:
+    """A decode step recorded as a HIP graph: static inputs, the graph, its logits."""
+
+    def __init__(self, inputs: torch.Tensor) -> None:
+        self.inputs = inputs
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+
+
 class StepRunner:
-    def __init__(self, model: Model, cache: CacheManager) -> None:
+    """Runs steps.  Steps in which every sequence brings exactly one token (decode
+    steps) are recorded once per shape as a HIP graph and replayed, so that a step
+    costs one copy of its inputs and one graph launch instead of hundreds of kernel
+    launches; this needs every part of the model to be `graph_safe` (no host-side
+    data in its forward) and is switched off otherwise."""
+
+    TABLE_ROUND = 64    # block tables of captured steps are padded to a multiple of this many pages
+    MAX_GRAPHS = 24
+
+    def __init__(self, model: Model, cache: CacheManager, use_graphs: bool = True) -> None:
         self.model = model
         self.cache = cache
         self.device = model.device
         self.vocab_size = model.plan.vocab_size
+        self.use_graphs = use_graphs and model.graph_safe
+        self._graphs: Dict[tuple, _CapturedStep] = {}
+        self.graph_replays = 0
 
     def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run one step.  Every entry's tokens must already be reserved in the
         cache (`cache.reserve(seq_id, len(token_ids))`), and they are the last
         tokens reserved.  Returns float32 logits [number of wanted places, vocab]
-        in the order of the entries and of each entry's `want`."""
+        in the order of the entries and of each entry's `want`.  The tensor may be
+        overwritten by the next call."""
         cache = self.cache
         ids: List[int] = []
         positions: List[int] = []
@@ -80,28 +102,43 @@ class StepRunner:
         if not ids:
             raise ValueError("a step needs at least one entry")
 
-        # one staging buffer, one copy to the device
         T, S = len(ids), len(seq_ids)
-        tables = []
-        for group in cache.groups:
-            per_seq = [cache.block_table(group.index, s) for s in seq_ids]
-            width = max(1, max(len(t) for t in per_seq))
-            tables.append((width, per_seq))
+        decode_only = self.use_graphs and T == S and (self.model.dtype == torch.float32 or S <= 64)
         decode_tokens = [q_starts[i] for i in range(S) if q_lens[i] == 1]
         tiles: List[int] = []
         for i in range(S):
             if q_lens[i] > 1:
                 for first in range(0, q_lens[i], TILE_TOKENS):
                     tiles += [i, q_starts[i] + first, min(TILE_TOKENS, q_lens[i] - first)]
-        total = 3 * T + S + len(rows) + len(decode_tokens) + len(tiles) + sum(S * w for w, _ in tables)
-        staging = torch.empty(total, dtype=torch.int32, pin_memory=True)
+        tables = []
+        for group in cache.groups:
+            per_seq = [cache.block_table(group.index, s) for s in seq_ids]
+            width = max(1, max(len(t) for t in per_seq))
+            if decode_only:
+                width = -(-width // self.TABLE_ROUND) * self.TABLE_ROUND
+            tables.append((width, per_seq))
+
+        # one staging buffer, one copy to the device
         flat: List[int] = ids + positions + tok_seq + slots + rows + decode_tokens + tiles
         for width, per_seq in tables:
             for table in per_seq:
                 flat.extend(table)
                 flat.extend([-1] * (width - len(table)))
-        staging.copy_(torch.tensor(flat, dtype=torch.int32))
-        dev = staging.to(self.device, non_blocking=True)
+        staging = torch.tensor(flat, dtype=torch.int32).pin_memory()
+
+        captured = None
+        if decode_only:
+            key = (S, len(rows), tuple(w for w, _ in tables))
+            captured = self._graphs.get(key)
+            if captured is None:
+                if len(self._graphs) >= self.MAX_GRAPHS:
+                    self._graphs.pop(next(iter(self._graphs)))
+                captured = self._graphs[key] = _CapturedStep(torch.empty(len(flat), dtype=torch.int32,
+                                                                         device=self.device))
+            captured.inputs.copy_(staging, non_blocking=True)
+            dev = captured.inputs
+        else:
+            dev = staging.to(self.device, non_blocking=True)
         off = 0
 
         def take(count):
@@ -121,4 +158,16 @@ class StepRunner:
                           cache=cache, seq_ids=seq_ids, q_starts=q_starts, q_lens=q_lens,
                           past_lens=past_lens, host_slots=slots, decode_tokens=d_decode,
                           prefill_tiles=d_tiles)
-        return self.model.forward(ctx, d_ids, d_rows)
+        if captured is None:
+            return self.model.forward(ctx, d_ids, d_rows)
+        if captured.graph is None:
+            # record the step: nothing runs during the recording, so replay it right away
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                captured.logits = self.model.forward(ctx, d_ids, d_rows)
+            captured.graph = graph
+        else:
+            self.model.forward_pass_count += 1
+        captured.graph.replay()
+        self.graph_replays += 1
+        return captured.logits

@@ -59,8 +59,10 @@ def _declare(lib) -> None:
         "pae_gemm_skinny": [I, P, L, P, L, P, P, I, I, I, I, I, L, P],
         "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
-        "pae_sample": [P, P, L, P, P, I, I, P],
-        "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P, P, P],
+        "pae_sample": [P, P, L, P, P, I, I, P, P, P, P],
+        "pae_sample_chunks": [I],
+        "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, P, P],
+        "pae_attn_decode_split": [],
         "pae_attn_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
     }
     for name, args in sig.items():
@@ -275,9 +277,6 @@ def paged_attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.T
         block_tables.shape[1], bs, T, nh, nkv, hd, float(scale), int(window), _stream()))
 
 
-DECODE_SPLIT = 256  # keys per workgroup of the decode kernel; fixed, so results do not depend on the batch
-
-
 def mfma_attention_supported(dtype: torch.dtype, nh: int, nkv: int, hd: int, bs: int) -> bool:
     """Shapes the matrix-core attention kernels take; others go through the generic kernel."""
     return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 256 and bs % 16 == 0 and nh // nkv <= 16
@@ -297,13 +296,13 @@ def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cac
     assert dec_tok.dtype == torch.int32 and positions.dtype == torch.int32 and tok_seq.dtype == torch.int32
     assert positions.numel() == q.shape[0] == tok_seq.numel()
     assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
-    max_splits = -(-block_tables.shape[1] * bs // DECODE_SPLIT)
+    max_splits = -(-block_tables.shape[1] * bs // library().pae_attn_decode_split())
     part_acc = torch.empty((n * nh * max_splits, hd), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n * nh * max_splits, 2), dtype=torch.float32, device=q.device)
     _check(library().pae_attn_decode_bf16(
         out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
         dec_tok.data_ptr(), n, positions.data_ptr(), tok_seq.data_ptr(), block_tables.data_ptr(),
-        block_tables.shape[1], bs, nh, nkv, hd, float(scale), int(window), DECODE_SPLIT,
+        block_tables.shape[1], bs, nh, nkv, hd, float(scale), int(window),
         part_acc.data_ptr(), part_ml.data_ptr(), _stream()))
 
 
@@ -337,5 +336,11 @@ def sample(tokens: torch.Tensor, logits: torch.Tensor, temperature: Optional[tor
     for t in (temperature, uniform):
         if t is not None:
             assert t.dtype == torch.float32 and t.numel() == R
+    chunks = library().pae_sample_chunks(V)
+    chunk_max = torch.empty(R * chunks, dtype=torch.float32, device=logits.device)
+    chunk_arg = torch.empty(R * chunks, dtype=torch.int32, device=logits.device)
+    chunk_sum = (torch.empty(R * chunks, dtype=torch.float64, device=logits.device)
+                 if temperature is not None else None)
     _check(library().pae_sample(tokens.data_ptr(), logits.data_ptr(), logits.stride(0), _ptr(temperature),
-                                _ptr(uniform), R, V, _stream()))
+                                _ptr(uniform), R, V, chunk_max.data_ptr(), chunk_arg.data_ptr(),
+                                _ptr(chunk_sum), _stream()))

@@ -24,6 +24,9 @@ from .linear import Linear
 
 @register_mixer("attention")
 class PagedAttention(Part):
+    @property
+    def graph_safe(self) -> bool:
+        return self.position.graph_safe
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         if spec.num_heads % spec.num_kv_heads:
@@ -33,6 +36,9 @@ class PagedAttention(Part):
         self.position = (build_part(POSITION_ENCODINGS, "position encoding", spec.position, dtype, device)
                          if spec.position is not None else
                          POSITION_ENCODINGS["none"](None, dtype, device))
+
+    def product_widths(self):
+        return [self.spec.hidden_size, self.spec.num_heads * self.spec.head_dim]
 
     def paged_spec(self):
         return PagedSpec(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)

@@ -67,6 +67,11 @@ class StepContext:
 class Part:
     """Base of all parts: holds its spec and the precision it computes in."""
 
+    # True when `forward` only launches work on the current stream with device-side
+    # data (nothing read from the context's host lists, no synchronisation): such a
+    # part can be recorded into a HIP graph and replayed with new inputs.
+    graph_safe = False
+
     def __init__(self, spec, dtype: torch.dtype, device) -> None:
         self.spec = spec
         self.dtype = dtype

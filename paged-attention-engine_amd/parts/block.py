@@ -19,6 +19,17 @@ class PreNormBlock:
         self.feed_forward_norm = build_part(NORMS, "norm", layer_spec.feed_forward_norm, dtype, device)
         self.feed_forward = build_part(FEED_FORWARDS, "feed-forward", layer_spec.feed_forward, dtype, device)
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for part, _ in self._named())
+
+    def product_widths(self):
+        """Inner dimensions of the block's matrix products (the skinny kernel wants multiples of 8)."""
+        out = []
+        for part, _ in self._named():
+            out += getattr(part, "product_widths", lambda: [])()
+        return out
+
     def _named(self):
         s = self.spec
         return ((self.mixer_norm, s.prefix + s.mixer_norm_prefix), (self.mixer, s.prefix + s.mixer_prefix),

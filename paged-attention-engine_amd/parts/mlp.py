@@ -13,10 +13,14 @@ from .linear import Linear
 
 @register_feed_forward("swiglu")
 class SwiGLU(Part):
+    graph_safe = True
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         if spec.activation != "silu":
             raise ValueError(f"activation '{spec.activation}' is not supported by the gated feed-forward")
+
+    def product_widths(self):
+        return [self.spec.hidden_size, self.spec.intermediate_size]
 
     def tensors(self, prefix):
         s = self.spec

@@ -18,6 +18,7 @@ from .base import Part, ResidualStream, register_norm
 
 @register_norm("rmsnorm")
 class RMSNorm(Part):
+    graph_safe = True
     def tensors(self, prefix):
         return {prefix + "weight": (self.spec.size,)}
 

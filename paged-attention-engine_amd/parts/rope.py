@@ -18,6 +18,7 @@ from .base import Part, register_position_encoding
 
 @register_position_encoding("neox_rope")
 class NeoxRope(Part):
+    graph_safe = True
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         rot = spec.rotary_dim
@@ -35,6 +36,7 @@ class NeoxRope(Part):
 
 @register_position_encoding("none")
 class NoPosition(Part):
+    graph_safe = True
     """No encoding: keys and values go to the cache as they are."""
 
     def encode_and_store(self, ctx, qkv, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
