@@ -210,12 +210,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 }
 
 // Adds a token's partials in split order and writes the output: one workgroup per
-// (token, kv head), launched after the kernel above.
+// (token, kv head), one thread per (head of the group, four features), launched after
+// the kernel above.  Kept small: it runs for microseconds.
 template <int HD, int TPW>
-__global__ __launch_bounds__(256) void attn_decode_merge_kernel(
-    bf16_t* __restrict__ out, int64_t out_stride, const float* __restrict__ part_acc,
-    const float* __restrict__ part_ml, int max_splits, const int* __restrict__ dec_tok,
-    const int* __restrict__ positions, int nh, int nkv, int window) {
+__global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
+                                         const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                         int max_splits, const int* __restrict__ dec_tok,
+                                         const int* __restrict__ positions, int nh, int nkv, int window) {
   constexpr int SPLIT = 64 * TPW;
   const int kvh = blockIdx.x;
   const int tok = dec_tok[blockIdx.y];
@@ -223,23 +224,28 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(
   const int start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int s_first = start / SPLIT, nsplits = pos / SPLIT - s_first + 1;
   const int g = nh / nkv;
-  const int64_t group_slot = ((int64_t)blockIdx.y * nkv + kvh) * max_splits;
-  for (int idx = threadIdx.x; idx < g * HD; idx += blockDim.x) {
-    const int c = idx / HD, d = idx % HD;
-    const int64_t slot0 = (group_slot + s_first) * g + c;  // consecutive splits are g slots apart
-    float m = NEG_BIG;
-#pragma unroll 8
-    for (int sp = 0; sp < nsplits; ++sp) m = fmaxf(m, part_ml[(slot0 + (int64_t)sp * g) * 2]);
-    float a = 0.f, l = 0.f;
-#pragma unroll 8
-    for (int sp = 0; sp < nsplits; ++sp) {
-      const int64_t slot = slot0 + (int64_t)sp * g;
-      const float f = exp2f(part_ml[slot * 2] - m);
-      a += f * part_acc[slot * HD + d];
-      l += f * part_ml[slot * 2 + 1];
-    }
-    out[(int64_t)tok * out_stride + (int64_t)(kvh * g + c) * HD + d] = __float2bfloat16(a / l);
+  const int item = threadIdx.x;  // (head in group, chunk of four features)
+  if (item >= g * (HD / 4)) return;
+  const int c = item / (HD / 4), d = (item % (HD / 4)) * 4;
+  const int64_t slot0 = (((int64_t)blockIdx.y * nkv + kvh) * max_splits + s_first) * g + c;
+  float m = NEG_BIG, l = 0.f;
+  f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int sp = 0; sp < nsplits; ++sp) {  // consecutive splits are g slots apart
+    const int64_t slot = slot0 + (int64_t)sp * g;
+    const float ms = part_ml[slot * 2], ls = part_ml[slot * 2 + 1];
+    const f32x4 v = *reinterpret_cast<const f32x4*>(part_acc + slot * HD + d);
+    const float m_new = fmaxf(m, ms);
+    const float f_old = exp2f(m - m_new), f = exp2f(ms - m_new);
+    a = a * f_old + v * f;
+    l = l * f_old + ls * f;
+    m = m_new;
   }
+  const float inv = 1.0f / l;
+  s16x4 w;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = bf16_bits(a[i] * inv);
+  *reinterpret_cast<s16x4*>(out + (int64_t)tok * out_stride + (int64_t)(kvh * g + c) * HD + d) = w;
 }
 
 // ------------------------------------------------------------------ prefill
@@ -360,7 +366,7 @@ extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q
       (float*)part_acc, (float*)part_ml, max_splits, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,     \
       (const bf16_t*)v_cache, dec_tok, positions, tok_seq, block_tables, max_blocks, bs, nh, nkv, scale_log2, \
       window);                                                                                               \
-  attn_decode_merge_kernel<HD, DECODE_TPW><<<merge_grid, 256, 0, stream>>>(                                  \
+  attn_decode_merge_kernel<HD, DECODE_TPW><<<merge_grid, (nh / nkv * (HD / 4) + 63) / 64 * 64, 0, stream>>>( \
       (bf16_t*)out, out_stride, (const float*)part_acc, (const float*)part_ml, max_splits, dec_tok, positions, \
       nh, nkv, window)
   FOR_HEAD_DIM(hd, CALL)

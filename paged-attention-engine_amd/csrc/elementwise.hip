@@ -50,11 +50,101 @@ __device__ __forceinline__ float pending_at(const void* delta, int parts, int64_
   return sum;
 }
 
-#define RMS_MAXP 8
-// EPT > 0: each thread keeps its EPT elements of the row in registers (hidden <= NT * EPT):
-// all loads are issued before the first is used and the row is read once.
-// EPT == 0: any width, two passes over the row.
-template <typename T, int NT, int EPT>
+// Sum over the wavefronts of a block of any size, in wavefront order.
+__device__ __forceinline__ float block_sum_any(float v, float* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / PAE_WAVE, nwaves = (blockDim.x + PAE_WAVE - 1) / PAE_WAVE;
+  if ((threadIdx.x & (PAE_WAVE - 1)) == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += scratch[w];
+  __syncthreads();
+  return total;
+}
+
+template <typename T>
+struct Vec4;
+template <>
+struct Vec4<float> {
+  typedef float4 type;
+  static __device__ __forceinline__ void unpack(const type& v, float (&f)[4]) { f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w; }
+  static __device__ __forceinline__ type pack(const float (&f)[4]) { return make_float4(f[0], f[1], f[2], f[3]); }
+};
+template <>
+struct Vec4<bf16_t> {
+  typedef uint2 type;  // four bfloat16
+  static __device__ __forceinline__ void unpack(const type& v, float (&f)[4]) {
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ type pack(const float (&f)[4]) {
+    bf16_t h[4] = {__float2bfloat16(f[0]), __float2bfloat16(f[1]), __float2bfloat16(f[2]), __float2bfloat16(f[3])};
+    return *reinterpret_cast<const type*>(h);
+  }
+};
+
+// Vector form for hidden % 4 == 0: a thread owns chunks of four elements; the launch
+// gives one chunk per thread up to a width of 4096, so a row is one round of loads.
+// The kernel is kept small on purpose: at a few rows it runs for microseconds and the
+// time goes to fetching its instructions.
+template <typename T>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const void* __restrict__ delta, int parts,
+                                       int64_t part_stride, const void* __restrict__ weight, int w_is_f32,
+                                       float eps, const int* __restrict__ rows, T* __restrict__ out, int hidden,
+                                       int write_residual) {
+  __shared__ float scratch[16];
+  typedef typename Vec4<T>::type vec_t;
+  const int b = blockIdx.x;
+  const int64_t src = rows ? rows[b] : b;
+  const int nvec = hidden / 4;
+  float4* res4 = reinterpret_cast<float4*>(residual + src * hidden);
+  const bool one_round = nvec <= (int)blockDim.x;  // every thread has at most one chunk: keep it in registers
+  float ss = 0.f;
+  float4 mine = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int v = threadIdx.x; v < nvec; v += blockDim.x) {
+    float4 r = res4[v];
+    if (delta) {
+      if (parts == 0) {
+        float d[4];
+        Vec4<T>::unpack(reinterpret_cast<const vec_t*>((const T*)delta + src * hidden)[v], d);
+        r.x += d[0]; r.y += d[1]; r.z += d[2]; r.w += d[3];
+      } else {
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);  // partial sums are added in order
+        for (int p = 0; p < parts; ++p) {
+          const float4 d = reinterpret_cast<const float4*>((const float*)delta + p * part_stride + src * hidden)[v];
+          sum.x += d.x; sum.y += d.y; sum.z += d.z; sum.w += d.w;
+        }
+        r.x += sum.x; r.y += sum.y; r.z += sum.z; r.w += sum.w;
+      }
+      if (write_residual) res4[v] = r;
+    }
+    ss += (r.x * r.x + r.y * r.y) + (r.z * r.z + r.w * r.w);
+    mine = r;
+  }
+  const float total = block_sum_any(ss, scratch);  // every thread of the block arrives here together
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+  for (int v = threadIdx.x; v < nvec; v += blockDim.x) {
+    float4 r = mine;
+    if (!one_round) {
+      r = res4[v];
+      if (delta && !write_residual)
+        for (int i = 0; i < 4; ++i) (&r.x)[i] += pending_at<T>(delta, parts, part_stride, src * hidden + 4 * v + i);
+    }
+    float w[4], o[4] = {r.x, r.y, r.z, r.w};
+    if (w_is_f32) {
+      const float4 wv = reinterpret_cast<const float4*>(weight)[v];
+      w[0] = wv.x; w[1] = wv.y; w[2] = wv.z; w[3] = wv.w;
+    } else {
+      Vec4<bf16_t>::unpack(reinterpret_cast<const uint2*>(weight)[v], w);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = w[i] * round_to<T>(o[i] * inv);
+    reinterpret_cast<vec_t*>(out + (int64_t)b * hidden)[v] = Vec4<T>::pack(o);
+  }
+}
+
+// Any width, two passes over the row.
+template <typename T, int NT>
 __global__ __launch_bounds__(NT) void add_rmsnorm_kernel(float* __restrict__ residual,
                                                          const void* __restrict__ delta, int parts,
                                                          int64_t part_stride, const void* __restrict__ weight,
@@ -65,62 +155,6 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_kernel(float* __restrict__ res
   const int64_t src = rows ? rows[b] : b;
   float* res = residual + src * hidden;
   T* dst = out + (int64_t)b * hidden;
-  if (EPT > 0) {
-    float r[EPT > 0 ? EPT : 1];
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < EPT; ++e) {
-      const int i = threadIdx.x + e * NT;
-      r[e] = i < hidden ? res[i] : 0.f;
-    }
-    if (delta) {
-      if (parts == 0) {
-#pragma unroll
-        for (int e = 0; e < EPT; ++e) {
-          const int i = threadIdx.x + e * NT;
-          if (i < hidden) r[e] += to_f32(((const T*)delta)[src * hidden + i]);
-        }
-      } else {
-        // partial sums are added in order; the first RMS_MAXP of them are loaded without
-        // branches (from a clamped address, dropped by a select) so that all are in flight at once
-        float psum[EPT > 0 ? EPT : 1];
-#pragma unroll
-        for (int e = 0; e < EPT; ++e) psum[e] = 0.f;
-#pragma unroll
-        for (int p = 0; p < RMS_MAXP; ++p) {
-          const float* part = (const float*)delta + (int64_t)(p < parts ? p : parts - 1) * part_stride + src * hidden;
-#pragma unroll
-          for (int e = 0; e < EPT; ++e) {
-            const int i = threadIdx.x + e * NT;
-            const float v = part[i < hidden ? i : 0];
-            psum[e] += (p < parts && i < hidden) ? v : 0.f;
-          }
-        }
-        for (int p = RMS_MAXP; p < parts; ++p)
-#pragma unroll
-          for (int e = 0; e < EPT; ++e) {
-            const int i = threadIdx.x + e * NT;
-            if (i < hidden) psum[e] += ((const float*)delta)[p * part_stride + src * hidden + i];
-          }
-#pragma unroll
-        for (int e = 0; e < EPT; ++e) r[e] += psum[e];
-      }
-    }
-#pragma unroll
-    for (int e = 0; e < EPT; ++e) {
-      const int i = threadIdx.x + e * NT;
-      if (write_residual && delta && i < hidden) res[i] = r[e];
-      ss += r[e] * r[e];
-    }
-    const float total = block_sum<NT / PAE_WAVE>(ss, scratch);
-    const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
-#pragma unroll
-    for (int e = 0; e < EPT; ++e) {
-      const int i = threadIdx.x + e * NT;
-      if (i < hidden) dst[i] = from_f32<T>(load_param(weight, w_is_f32, i) * round_to<T>(r[e] * inv));
-    }
-    return;
-  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += NT) {
     float r = res[i];
@@ -145,23 +179,25 @@ extern "C" int pae_add_rmsnorm(int dtype, void* residual, const void* delta, int
   PAE_REQUIRE(num_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d H=%d", num_rows, hidden);
   PAE_REQUIRE(!(rows && write_residual), "add_rmsnorm: a row gather may not write the residual back");
   if (num_rows == 0) return 0;
-#define RMS_LAUNCH(T, EPT)                                                                                  \
-  add_rmsnorm_kernel<T, 256, EPT><<<num_rows, 256, 0, stream>>>((float*)residual, delta, parts, part_stride, \
+  const bool vec = hidden % 4 == 0;
+  int threads = ((hidden / 4 + PAE_WAVE - 1) / PAE_WAVE) * PAE_WAVE;
+  threads = threads > 1024 ? 1024 : threads;
+#define RMS_LAUNCH(T)                                                                                         \
+  if (vec)                                                                                                    \
+    add_rmsnorm_vec_kernel<T><<<num_rows, threads, 0, stream>>>((float*)residual, delta, parts, part_stride,  \
                                                                 weight, w_is_f32, eps, rows, (T*)out, hidden, \
-                                                                write_residual)
-#define RMS_BY_WIDTH(T)                          \
-  if (hidden <= 256 * 2) RMS_LAUNCH(T, 2);       \
-  else if (hidden <= 256 * 8) RMS_LAUNCH(T, 8);  \
-  else if (hidden <= 256 * 32) RMS_LAUNCH(T, 32); \
-  else RMS_LAUNCH(T, 0)
+                                                                write_residual);                              \
+  else                                                                                                        \
+    add_rmsnorm_kernel<T, 256><<<num_rows, 256, 0, stream>>>((float*)residual, delta, parts, part_stride,     \
+                                                             weight, w_is_f32, eps, rows, (T*)out, hidden,    \
+                                                             write_residual)
   if (dtype == PAE_F32) {
-    RMS_BY_WIDTH(float);
+    RMS_LAUNCH(float);
   } else if (dtype == PAE_BF16) {
-    RMS_BY_WIDTH(bf16_t);
+    RMS_LAUNCH(bf16_t);
   } else {
     return pae_fail("add_rmsnorm: unknown dtype code %d", dtype);
   }
-#undef RMS_BY_WIDTH
 #undef RMS_LAUNCH
   return pae_check_launch("add_rmsnorm");
 }
@@ -203,47 +239,44 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, in
                                      const int* __restrict__ positions, const int* __restrict__ tok_seq,
                                      const int* __restrict__ block_tables, int max_blocks, int bs,
                                      T* __restrict__ k_cache, T* __restrict__ v_cache, int write_kv) {
+  // One item per (head, rotated pair), then per (kv head, value feature): every thread's
+  // loads are independent of the others' stores, so a token is one round of memory traffic.
   const int t = blockIdx.x;
   const int pos = positions[t];
   T* row = qkv + (int64_t)t * row_stride;
-  T* q = row;
-  T* k = row + (int64_t)nh * hd;
-  T* v = k + (int64_t)nkv * hd;
+  const T* k = row + (int64_t)nh * hd;
+  const T* v = k + (int64_t)nkv * hd;
   int64_t page_base = 0;  // element offset of (block, kv head 0) in either pool
   const int64_t head_step = (int64_t)bs * hd;
   const int off = pos % bs;
   if (write_kv) page_base = (int64_t)block_tables[(int64_t)tok_seq[t] * max_blocks + pos / bs] * nkv * head_step;
-  const int64_t slot_base = page_base + (int64_t)off * hd;  // key row of this token, kv head 0
   const int half = rot / 2;
-  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+  const int rotated_heads = nh + (write_kv ? nkv : 0);
+  for (int idx = threadIdx.x; idx < rotated_heads * half; idx += blockDim.x) {
+    const int h = idx / half, i = idx % half;
     float s = 0.f, c = 1.f;
     if (inv_freq) sincosf((float)pos * inv_freq[i], &s, &c);
-    for (int h = 0; h < nh; ++h) {
-      const float a = to_f32(q[h * hd + i]), b = to_f32(q[h * hd + i + half]);
-      q[h * hd + i] = from_f32<T>(a * c - b * s);
-      q[h * hd + i + half] = from_f32<T>(b * c + a * s);
-    }
-    if (write_kv) {
-      for (int h = 0; h < nkv; ++h) {
-        const float a = to_f32(k[h * hd + i]), b = to_f32(k[h * hd + i + half]);
-        T* dst = k_cache + slot_base + h * head_step;
-        dst[i] = from_f32<T>(a * c - b * s);
-        dst[i + half] = from_f32<T>(b * c + a * s);
-      }
+    const float a = to_f32(row[h * hd + i]), b = to_f32(row[h * hd + i + half]);
+    const T lo = from_f32<T>(a * c - b * s), hi = from_f32<T>(b * c + a * s);
+    if (h < nh) {  // queries are rotated in place
+      row[h * hd + i] = lo;
+      row[h * hd + i + half] = hi;
+    } else {       // keys go to [block][kv head][offset][feature]
+      T* dst = k_cache + page_base + (h - nh) * head_step + (int64_t)off * hd;
+      dst[i] = lo;
+      dst[i + half] = hi;
     }
   }
-  if (write_kv) {
-    const int tail = hd - rot;  // features of a key beyond the rotated ones pass through
-    for (int idx = threadIdx.x; idx < nkv * tail; idx += blockDim.x) {
-      const int h = idx / tail, i = rot + idx % tail;
-      k_cache[slot_base + h * head_step + i] = k[h * hd + i];
-    }
-    // values are stored transposed within a page: [kv head][feature][offset in page]
-    const int64_t v_base = page_base + off;
-    for (int idx = threadIdx.x; idx < nkv * hd; idx += blockDim.x) {
-      const int h = idx / hd, i = idx % hd;
-      v_cache[v_base + h * head_step + (int64_t)i * bs] = v[h * hd + i];
-    }
+  if (!write_kv) return;
+  const int tail = hd - rot;  // features of a key beyond the rotated ones pass through
+  for (int idx = threadIdx.x; idx < nkv * tail; idx += blockDim.x) {
+    const int h = idx / tail, i = rot + idx % tail;
+    k_cache[page_base + h * head_step + (int64_t)off * hd + i] = k[h * hd + i];
+  }
+  // values are stored transposed within a page: [block][kv head][feature][offset]
+  for (int idx = threadIdx.x; idx < nkv * hd; idx += blockDim.x) {
+    const int h = idx / hd, i = idx % hd;
+    v_cache[page_base + h * head_step + (int64_t)i * bs + off] = v[h * hd + i];
   }
 }
 
@@ -258,11 +291,11 @@ extern "C" int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int n
               "rope_kv_write: cache write needs tables and pools");
   if (num_tokens <= 0) return 0;
   if (dtype == PAE_F32)
-    rope_kv_write_kernel<float><<<num_tokens, 128, 0, stream>>>(
+    rope_kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>(
         (float*)qkv, row_stride, nh, nkv, hd, rot, inv_freq, positions, tok_seq, block_tables, max_blocks, bs,
         (float*)k_cache, (float*)v_cache, write_kv);
   else if (dtype == PAE_BF16)
-    rope_kv_write_kernel<bf16_t><<<num_tokens, 128, 0, stream>>>(
+    rope_kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, nh, nkv, hd, rot, inv_freq, positions, tok_seq, block_tables, max_blocks, bs,
         (bf16_t*)k_cache, (bf16_t*)v_cache, write_kv);
   else

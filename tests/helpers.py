@@ -1,6 +1,6 @@
 """Tiny configurations, model folders and tolerances shared by the tests.
 
-The three tiny configurations differ in every size and option: head counts and
+The tiny configurations differ in every size and option: head counts and
 groups, sizes that are no power of two, number of layers, vocabulary, eps,
 rope base, tying of the head, norm weights and, in the third, windows.
 """
@@ -29,9 +29,18 @@ TINY_C = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=4, hidden_si
               use_sliding_window=True, sliding_window=24, max_window_layers=2,
               max_position_embeddings=512, hidden_act="silu")
 
+# a shape the matrix-core attention kernels take (head_dim 32, pages of 16), five query heads on
+# one key/value head, a window on the second of two layers
+TINY_D = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=2, hidden_size=160,
+              num_attention_heads=5, num_key_value_heads=1, head_dim=32, intermediate_size=400,
+              vocab_size=1111, rope_theta=200000.0, rms_norm_eps=2e-6, tie_word_embeddings=False,
+              use_sliding_window=True, sliding_window=40, max_window_layers=1,
+              max_position_embeddings=1024, hidden_act="silu")
+
 TINY = {"A": (TINY_A, dict(seed=0, norm_std=0.0, block_size=16)),
         "B": (TINY_B, dict(seed=1, norm_std=0.1, block_size=8)),
-        "C": (TINY_C, dict(seed=2, norm_std=0.1, block_size=16))}
+        "C": (TINY_C, dict(seed=2, norm_std=0.1, block_size=16)),
+        "D": (TINY_D, dict(seed=3, norm_std=0.05, block_size=16))}
 
 
 def make_model_folder(tmp_path, name: str) -> str:

@@ -14,7 +14,7 @@ from tests import helpers
 from tests.plain import qwen2_plain as plain
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_config_reads_every_key(name):
     raw = helpers.TINY[name][0]
     cfg = pae.read_config_dict(raw)

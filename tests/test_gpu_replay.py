@@ -127,7 +127,7 @@ def run_trace(folder, dtype, out_dir, max_tokens, block_size, records):
     assert proc.wait(timeout=60) == 0
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_replay_schedules_agree_with_the_plain_implementation(tmp_path, name, dtype):
     folder = helpers.make_model_folder(tmp_path, name)
