@@ -151,6 +151,7 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=FULL_LAYERS)
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
+    parser.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this engine has no multi-GPU path (run with --gpus 1)")
@@ -164,6 +165,12 @@ def main() -> int:
     elem = 2 if args.dtype == "bfloat16" else 4
     model = build_model(cfg, args.dtype)
 
+    if args.prefill_only:
+        pre_s = prefill_run(model, cfg, 2048, repeats=max(3, args.steps))
+        print(json.dumps({"metric": "prefill tok/s at 2,048 tokens (Qwen2.5-1.5B shape)", "value": round(2048 / pre_s, 1),
+                          "unit": "tokens/s", "ms": round(pre_s * 1e3, 3), "dtype": args.dtype,
+                          "frac": round(prefill_flops(cfg, 2048) / pre_s / PEAK_FLOPS[args.dtype], 4)}))
+        return 0
     step_s, tokens_held = decode_run(model, cfg, args.batch, args.ctx, args.steps, args.warmup)
     value = args.batch / step_s
     step_bytes = weight_bytes(cfg, elem) + kv_bytes(cfg, tokens_held, elem)

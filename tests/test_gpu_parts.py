@@ -1,0 +1,292 @@
+"""Each part alone against the plain functions, and the framework's generality: a toy
+mixer with state of its own, a toy position encoding and a toy architecture whose schedule
+names a layer twice and lets a stop read another stop's cache are registered here, built
+and stepped (in portions, several sequences at once) without touching the framework's files."""
+
+import math
+
+import pytest
+import torch
+
+import paged_attention_engine_amd as pae
+from paged_attention_engine_amd import parts as P
+from paged_attention_engine_amd.cache import CacheManager, PagedSpec, StateSpec
+from paged_attention_engine_amd.config import (FeedForwardSpec, LayerSpec, MixerSpec, ModelPlan, NormSpec, PartSpec,
+                                               PositionSpec, ScheduleEntry)
+from tests.plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+
+
+def make_ctx(cache, dtype, seq_ids, q_lens):
+    """A step context for sequences that have already reserved `q_lens` new tokens."""
+    positions, tok_seq, q_starts, past = [], [], [], []
+    for row, (s, n) in enumerate(zip(seq_ids, q_lens)):
+        held = cache.num_tokens(s)
+        q_starts.append(len(positions))
+        past.append(held - n)
+        positions += list(range(held - n, held))
+        tok_seq += [row] * n
+    tables = {}
+    for group in cache.groups:
+        rows = [cache.block_table(group.index, s) for s in seq_ids]
+        width = max(len(r) for r in rows)
+        tables[group.index] = torch.tensor([list(r) + [-1] * (width - len(r)) for r in rows], dtype=torch.int32, device=DEV)
+    slots = [cache.slot_of(s) for s in seq_ids]
+    dec = [q_starts[i] for i, n in enumerate(q_lens) if n == 1]
+    tiles = [[i, q_starts[i] + f, min(32, n - f)] for i, n in enumerate(q_lens) if n > 1 for f in range(0, n, 32)]
+    return P.StepContext(
+        dtype=dtype, device=torch.device(DEV), num_tokens=len(positions), num_seqs=len(seq_ids),
+        positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
+        tok_seq=torch.tensor(tok_seq, dtype=torch.int32, device=DEV), block_tables=tables,
+        slots=torch.tensor(slots, dtype=torch.int32, device=DEV), cache=cache, seq_ids=list(seq_ids),
+        q_starts=q_starts, q_lens=list(q_lens), past_lens=past, host_slots=slots,
+        decode_tokens=torch.tensor(dec, dtype=torch.int32, device=DEV),
+        prefill_tiles=torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 3))
+
+
+# ------------------------------------------------------------------ built-in parts, one at a time
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_norm_part(dtype):
+    spec = NormSpec(size=200, eps=3e-6)
+    part = P.build_part(P.NORMS, "norm", spec, DT[dtype], DEV)
+    assert part.tensors("x.") == {"x.weight": (200,)}
+    w = 1 + 0.1 * torch.randn(200)
+    part.bind("x.", {"x.weight": w.to(DT[dtype])})
+    res = torch.randn(6, 200)
+    branch = torch.randn(6, 200).to(DT[dtype])
+    stream = P.ResidualStream(res.to(DEV))
+    stream.pending = branch.to(DEV)
+    out = part.forward(stream)
+    want = plain.rms_norm((res + branch.float()).double(), w.to(DT[dtype]).double(), 3e-6)
+    assert stream.pending is None and torch.allclose(stream.residual.cpu(), res + branch.float(), atol=1e-6)
+    assert (out.double().cpu() - want).abs().max() <= TOL[dtype] * 4
+    stream.pending = branch.to(DEV)
+    rows = part.forward(stream, torch.tensor([5, 2], dtype=torch.int32, device=DEV))
+    want2 = plain.rms_norm((res + 2 * branch.float()).double(), w.to(DT[dtype]).double(), 3e-6)[[5, 2]]
+    assert stream.pending is not None and (rows.double().cpu() - want2).abs().max() <= TOL[dtype] * 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden,inter", [(96, 208), (72, 200)])  # the second is not a multiple of 16
+def test_feed_forward_part(dtype, hidden, inter):
+    torch.manual_seed(0)
+    spec = FeedForwardSpec(hidden_size=hidden, intermediate_size=inter)
+    part = P.build_part(P.FEED_FORWARDS, "feed-forward", spec, DT[dtype], DEV)
+    names = part.tensors("m.mlp.")
+    assert names == {"m.mlp.gate_proj.weight": (inter, hidden), "m.mlp.up_proj.weight": (inter, hidden),
+                     "m.mlp.down_proj.weight": (hidden, inter)}
+    w = {n: (torch.randn(shape) * 0.2).to(DT[dtype]) for n, shape in names.items()}
+    part.bind("m.mlp.", w)
+    for rows in (5, 70):  # the skinny products and the library's
+        x = torch.randn(rows, hidden).to(DT[dtype])
+        got = part.forward(None, x.to(DEV))
+        got = got.sum(0) if got.dim() == 3 else got  # float32 partial sums are added by the next norm
+        want = plain.swiglu_mlp({k: v.double() for k, v in w.items()}, "m.", x.double())
+        assert (got.double().cpu() - want).abs().max() <= TOL[dtype] * max(1.0, float(want.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,window,bs", [(4, 2, 16, None, 8), (6, 2, 32, 20, 16), (5, 1, 64, None, 16)])
+def test_attention_part_in_portions(dtype, nh, nkv, hd, window, bs):
+    """The mixer alone, two sequences at once, the first in portions of 9, 1 and 30 tokens."""
+    torch.manual_seed(1)
+    hidden = 80
+    spec = MixerSpec(hidden_size=hidden, num_heads=nh, num_kv_heads=nkv, head_dim=hd, scale=hd ** -0.5,
+                     qkv_bias=True, window=window, position=PositionSpec(rotary_dim=hd, theta=12345.0))
+    part = P.build_part(P.MIXERS, "mixer", spec, DT[dtype], DEV)
+    names = part.tensors("a.self_attn.")
+    w = {n: (torch.randn(shape) * 0.15).to(DT[dtype]) for n, shape in names.items()}
+    part.bind("a.self_attn.", w)
+    cache = CacheManager([part.paged_spec()], [None], bs, 24, 4, DT[dtype], DEV)
+    cfg = dict(num_attention_heads=nh, num_key_value_heads=nkv, head_dim=hd, rope_theta=12345.0)
+    xs = {0: torch.randn(40, hidden).to(DT[dtype]), 1: torch.randn(17, hidden).to(DT[dtype])}
+    want = {s: plain.self_attention({k: v.double() for k, v in w.items()}, "a.", cfg, x.double(),
+                                    torch.arange(x.shape[0]), window) for s, x in xs.items()}
+    for s in xs:
+        cache.create_sequence(s)
+    done = {0: 0, 1: 0}
+    for step in ([(0, 9), (1, 17)], [(0, 1)], [(0, 30)]):
+        for s, n in step:
+            cache.reserve(s, n)
+        ctx = make_ctx(cache, DT[dtype], [s for s, _ in step], [n for _, n in step])
+        x = torch.cat([xs[s][done[s]:done[s] + n] for s, n in step]).to(DEV)
+        got = part.forward(ctx, x)
+        got = got.sum(0) if got.dim() == 3 else got
+        ref = torch.cat([want[s][done[s]:done[s] + n] for s, n in step])
+        assert (got.double().cpu() - ref).abs().max() <= TOL[dtype] * max(1.0, float(ref.abs().max()))
+        for s, n in step:
+            done[s] += n
+            cache.release_passed(s)
+
+
+# ------------------------------------------------------------------ toy parts registered by this test
+@P.register_mixer("toy_decay")
+class DecayMixer(P.Part):
+    """y_t = s_t, s_t = decay * s_{t-1} + W x_t: a mixer that keeps a vector per request
+    instead of keys and values.  Written with library calls and host loops (a test part)."""
+
+    def state_spec(self):
+        return StateSpec((self.spec.hidden_size,), torch.float32)
+
+    def tensors(self, prefix):
+        return {prefix + "in.weight": (self.spec.hidden_size, self.spec.hidden_size)}
+
+    def bind(self, prefix, weights):
+        self.w = weights[prefix + "in.weight"].to(device=self.device, dtype=torch.float32)
+
+    def forward(self, ctx, x):
+        state = ctx.cache.state_of(ctx.cache_entry)
+        u = x.float() @ self.w.t()
+        out = torch.empty_like(u)
+        for start, n, slot in zip(ctx.q_starts, ctx.q_lens, ctx.host_slots):
+            s = state[slot]
+            for t in range(start, start + n):
+                s = self.spec.decay * s + u[t]
+                out[t] = s
+            state[slot] = s
+        return out.to(x.dtype)
+
+
+@P.register_position_encoding("toy_shift")
+class ShiftEncoding(P.Part):
+    """Adds position / 100 to the first feature of every query and key head (a toy)."""
+
+    def encode_and_store(self, ctx, qkv, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
+        from paged_attention_engine_amd.kernels import lib as K
+        heads = qkv.view(qkv.shape[0], -1, hd)
+        rotated = nh + (nkv if k_cache is not None else 0)
+        heads[:, :rotated, 0] += (ctx.positions.float() / 100.0).to(qkv.dtype)[:, None]
+        if k_cache is not None:
+            K.rope_kv_write(qkv, nh, nkv, hd, 0, None, ctx.positions, ctx.tok_seq, block_table, block_size,
+                            k_cache, v_cache)
+
+
+from dataclasses import dataclass
+
+
+@dataclass(frozen=True)
+class DecaySpec(PartSpec):
+    hidden_size: int = 0
+    decay: float = 0.5
+    kind: str = "toy_decay"
+
+
+class ToyConfig:
+    """config.json of a made-up architecture: attention, a decay mixer, attention again through
+    the first stop's weights, and a stop that reads the first stop's cache."""
+
+    def __init__(self, cfg):
+        self.cfg = dict(cfg)
+
+    def to_json_dict(self):
+        return dict(self.cfg)
+
+    def plan(self):
+        c = self.cfg
+        H, hd = c["hidden_size"], c["head_dim"]
+        norm = NormSpec(size=H, eps=c["eps"])
+        attn = MixerSpec(hidden_size=H, num_heads=c["heads"], num_kv_heads=c["kv_heads"], head_dim=hd,
+                         scale=hd ** -0.5, qkv_bias=False, position=PositionSpec(kind="toy_shift"))
+        ffn = FeedForwardSpec(hidden_size=H, intermediate_size=c["inter"])
+        layers = (LayerSpec("layers.0.", attn, ffn, norm, norm), LayerSpec("layers.1.", DecaySpec(hidden_size=H, decay=c["decay"]), ffn, norm, norm))
+        schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(0, cache_from=0), ScheduleEntry(1))
+        return ModelPlan("ToyForCausalLM", H, c["vocab"], layers, schedule, norm, "embed.weight", "head.weight", "final_norm.")
+
+
+pae.register_architecture("ToyForCausalLM", ToyConfig)
+TOY = dict(architectures=["ToyForCausalLM"], hidden_size=48, head_dim=16, heads=3, kv_heads=1, inter=64, vocab=97,
+           eps=1e-5, decay=0.6)
+
+
+def toy_plain_logits(w, c, ids):
+    """The toy architecture written out plainly (float64, whole sequence, no cache)."""
+    x = w["embed.weight"][ids].double()
+    n = len(ids)
+    pos = torch.arange(n, dtype=torch.float64)
+    kv_of_stop0 = None
+
+    def attention(prefix, h, borrowed=None):
+        nh, nkv, hd = c["heads"], c["kv_heads"], c["head_dim"]
+        q = plain.split_heads(plain.linear(h, w[prefix + "q_proj.weight"].double()), nh, hd).clone()
+        q[:, :, 0] += pos / 100.0
+        if borrowed is None:
+            k = plain.split_heads(plain.linear(h, w[prefix + "k_proj.weight"].double()), nkv, hd).clone()
+            v = plain.split_heads(plain.linear(h, w[prefix + "v_proj.weight"].double()), nkv, hd)
+            k[:, :, 0] += pos / 100.0
+        else:
+            k, v = borrowed
+        out = plain.attention(q, k, v, hd ** -0.5)
+        return plain.linear(plain.merge_heads(out), w[prefix + "o_proj.weight"].double()), (k, v)
+
+    def decay(prefix, h):
+        u = h @ w[prefix + "in.weight"].double().t()
+        s, rows = torch.zeros(u.shape[1], dtype=torch.float64), []
+        for t in range(n):
+            s = c["decay"] * s + u[t]
+            rows.append(s)
+        return torch.stack(rows)
+
+    for stop, (layer, borrow) in enumerate(((0, False), (1, False), (0, False), (0, True), (1, False))):
+        p = f"layers.{layer}."
+        h = plain.rms_norm(x, w[p + "input_layernorm.weight"].double(), c["eps"])
+        if layer == 0:
+            y, kv = attention(p + "self_attn.", h, kv_of_stop0 if borrow else None)
+            if stop == 0:
+                kv_of_stop0 = kv
+        else:
+            y = decay(p + "self_attn.", h)
+        x = x + y
+        h = plain.rms_norm(x, w[p + "post_attention_layernorm.weight"].double(), c["eps"])
+        x = x + plain.swiglu_mlp({k: v.double() for k, v in w.items()}, p, h)
+    return plain.linear(plain.rms_norm(x, w["final_norm.weight"].double(), c["eps"]), w["head.weight"].double())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
+    assert "ToyForCausalLM" in pae.known_architectures()
+    config = pae.read_config_dict(TOY)
+    folder = pae.write_model_folder(config, 5, str(tmp_path / "toy"), std=0.08)
+    model = pae.load_model(folder, dtype)
+    assert not model.graph_safe  # the toy parts run host loops: steps are launched eagerly
+    paged, states = model.cache_specs()
+    assert [p is not None for p in paged] == [True, False, True, False, False]  # stop 3 borrows stop 0's cache
+    assert [s is not None for s in states] == [False, True, False, False, True]
+    cache = model.new_cache(8, 32, 3)
+    assert len(cache.groups) == 1 and cache.groups[0].entries == [0, 2]
+    runner = pae.StepRunner(model, cache)
+    weights = pae.load_weights(folder, model.expected_tensors())
+    w = {k: v.float() for k, v in weights.items()}
+    gen = torch.Generator().manual_seed(2)
+    seqs = {s: torch.randint(0, 97, (n,), generator=gen).tolist() for s, n in ((0, 30), (1, 19), (2, 7))}
+    want = {s: toy_plain_logits(w, TOY, ids).float() for s, ids in seqs.items()}
+    tol = helpers_tol(dtype, max(float(v.abs().max()) for v in want.values()))
+    done = {s: 0 for s in seqs}
+    for s in seqs:
+        assert cache.create_sequence(s)
+    plans = ([(0, 11), (1, 19)], [(0, 1), (2, 2)], [(0, 2), (2, 5)], [(0, 16)])
+    for plan in plans:
+        entries = []
+        for s, n in plan:
+            cache.reserve(s, n)
+            entries.append(pae.StepEntry(s, tuple(seqs[s][done[s]:done[s] + n]), tuple(range(n))))
+        got = runner.run(entries).cpu()
+        ref = torch.cat([want[s][done[s]:done[s] + n] for s, n in plan])
+        assert float((got - ref).abs().max()) <= tol
+        for s, n in plan:
+            done[s] += n
+    # a freed request's state slot is zeroed for the next one: the same tokens give the same logits
+    cache.free_sequence(2)
+    assert cache.create_sequence(7)
+    cache.reserve(7, 7)
+    again = runner.run([pae.StepEntry(7, tuple(seqs[2]), tuple(range(7)))]).cpu()
+    assert float((again - want[2]).abs().max()) <= tol
+
+
+def helpers_tol(dtype, top):
+    from tests import helpers
+    ref = torch.tensor(top)
+    return helpers.fp32_atol(ref) * 4 if dtype == "float32" else helpers.bf16_atol(ref)
