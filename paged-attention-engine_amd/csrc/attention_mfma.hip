@@ -392,3 +392,185 @@ extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* 
 #undef CALL
   return pae_check_launch("attn_prefill");
 }
+
+// ------------------------------------------------------------------ prefill, long runs
+// One workgroup per (up to 128 consecutive tokens of a sequence, query head); each of
+// its four wavefronts owns 32 of the tokens.  Keys and values of BN keys at a time are
+// staged in LDS by the whole workgroup (the next tile is fetched into registers while
+// the current one is used) and every wavefront multiplies them with its own queries:
+//   S^T[32 keys x 32 tokens] = K * Q^T             (MFMA 32x32x16, k = hd)
+//   O^T[32 features x 32 tokens] += V^T * P^T      (MFMA 32x32x16, k = 16 keys)
+// The accumulator of S^T holds, per lane (token = lane % 32, half = lane / 32), keys
+// 8 j + 4 half + i of each 32-key block; two such groups of four are the 8 k-slots of a
+// lane in the second product, whose A operand reads the values of exactly those keys.
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+template <int HD, int BN>
+__global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
+    bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ tiles,
+    const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int bs, int nh,
+    int nkv, float scale_log2, int window) {
+  constexpr int KS = HD + 8;   // row stride of the key tile in LDS (elements), padded against bank conflicts
+  constexpr int VS = BN + 8;   // row stride of the transposed value tile
+  constexpr int PAGES = BN / 16;
+  constexpr int KCH = (16 * HD / 8 + 255) / 256;  // 16-byte chunks per thread and page
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[BN * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[HD * VS];
+
+  const int tid = threadIdx.x, wave = tid / PAE_WAVE, lane = tid % PAE_WAVE;
+  const int col = lane % 32, half = lane / 32;
+  const int head = blockIdx.y, kvh = head / (nh / nkv);
+  const int seq_row = tiles[blockIdx.x * 3], tok0 = tiles[blockIdx.x * 3 + 1], ntok = tiles[blockIdx.x * 3 + 2];
+  const int* table = block_tables + (int64_t)seq_row * max_blocks;
+  const int pos0 = positions[tok0];
+  const int c = wave * 32 + col;          // this lane's token within the tile
+  const bool live = c < ntok;
+  const int pos = live ? pos0 + c : -1;   // a dead column sees no key
+  const int start = (live && window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int wave_hi = min(pos0 + wave * 32 + 31, pos0 + ntok - 1);  // last position of this wavefront
+  const bool wave_live = wave * 32 < ntok;
+  const int lo = (window > 0 && pos0 - window + 1 > 0) ? (pos0 - window + 1) / BN * BN : 0;
+  const int hi = pos0 + ntok - 1;
+
+  // queries: B operand, lane holds token `col`, features 16 ks + 8 half .. + 7
+  bf16x8 qf[HD / 16];
+  {
+    const bf16_t* qrow = q + (int64_t)(tok0 + (live ? c : 0)) * q_stride + (int64_t)head * HD;
+#pragma unroll
+    for (int ks = 0; ks < HD / 16; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + 16 * ks + 8 * half);
+  }
+  f32x16 acc[HD / 32];
+#pragma unroll
+  for (int t = 0; t < HD / 32; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+  float m = NEG_BIG, l = 0.f;
+
+  const int page_elems = bs * HD;
+  // staging registers: per page, this thread's 16-byte chunks of the key page and of the value page
+  bf16x8 kreg[PAGES][KCH], vreg[PAGES][KCH];
+  auto fetch = [&](int key0) {
+#pragma unroll
+    for (int p = 0; p < PAGES; ++p) {
+      const int key = key0 + 16 * p;
+      const int kc = key <= hi ? key : key0;  // pages past the end repeat the first one (never used)
+      const int64_t base = ((int64_t)table[kc / bs] * nkv + kvh) * page_elems;
+      const bf16_t* kp = k_cache + base + (int64_t)(kc % bs) * HD;  // [16 keys][HD], contiguous
+      const bf16_t* vp = v_cache + base + kc % bs;                  // [HD][bs]: 16 keys of each feature
+#pragma unroll
+      for (int ch = 0; ch < KCH; ++ch) {
+        const int idx = tid + 256 * ch;  // chunk index within the page: 16 * HD / 8 chunks
+        if (idx < 16 * HD / 8) {
+          kreg[p][ch] = *reinterpret_cast<const bf16x8*>(kp + idx * 8);
+          const int d = idx / 2, part = idx % 2;  // feature, which 8 of the 16 keys
+          vreg[p][ch] = *reinterpret_cast<const bf16x8*>(vp + (int64_t)d * bs + 8 * part);
+        }
+      }
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int p = 0; p < PAGES; ++p)
+#pragma unroll
+      for (int ch = 0; ch < KCH; ++ch) {
+        const int idx = tid + 256 * ch;
+        if (idx < 16 * HD / 8) {
+          const int key = idx / (HD / 8), kchunk = idx % (HD / 8);
+          *reinterpret_cast<bf16x8*>(k_lds + (16 * p + key) * KS + 8 * kchunk) = kreg[p][ch];
+          const int d = idx / 2, part = idx % 2;
+          *reinterpret_cast<bf16x8*>(v_lds + d * VS + 16 * p + 8 * part) = vreg[p][ch];
+        }
+      }
+  };
+
+  fetch(lo);
+  for (int key0 = lo; key0 <= hi; key0 += BN) {
+    __syncthreads();  // the previous tile has been read by every wavefront
+    stage();
+    __syncthreads();
+    if (key0 + BN <= hi) fetch(key0 + BN);
+    if (!wave_live || key0 > wave_hi) continue;  // nothing for this wavefront in the tile (causal)
+#pragma unroll
+    for (int kb = 0; kb < BN / 32; ++kb) {
+      f32x16 s;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < HD / 16; ++ks) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(k_lds + (32 * kb + col) * KS + 16 * ks + 8 * half);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s, 0, 0, 0);
+      }
+      float mx = NEG_BIG;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = key0 + 32 * kb + 8 * (v / 4) + 4 * half + v % 4;
+        s[v] = (key <= pos && key >= start) ? s[v] * scale_log2 : -INFINITY;
+        mx = fmaxf(mx, s[v]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, PAE_WAVE));
+      const float m_new = fmaxf(m, mx);
+      const float alpha = exp2f(m - m_new);
+      m = m_new;
+      float psum = 0.f;
+      bf16x8 pb[2];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float p = exp2f(s[v] - m_new);
+        psum += p;
+        pb[v / 8][v % 8] = (__bf16)p;
+      }
+      l = l * alpha + psum;
+#pragma unroll
+      for (int t = 0; t < HD / 32; ++t) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] *= alpha;
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          // values of keys 16 st + 4 half + (0..3) and 16 st + 8 + 4 half + (0..3) of this block, feature 32 t + col
+          const bf16_t* vrow = v_lds + (32 * t + col) * VS + 32 * kb + 16 * st + 4 * half;
+          bf16x8 vf;
+          const s16x4 a = *reinterpret_cast<const s16x4*>(vrow);
+          const s16x4 b = *reinterpret_cast<const s16x4*>(vrow + 8);
+          s16x4* dst = reinterpret_cast<s16x4*>(&vf);
+          dst[0] = a;
+          dst[1] = b;
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[st], acc[t], 0, 0, 0);
+        }
+      }
+    }
+  }
+  l += __shfl_xor(l, 32, PAE_WAVE);
+  if (!live) return;
+  const float inv = 1.0f / l;
+  bf16_t* o = out + (int64_t)(tok0 + c) * out_stride + (int64_t)head * HD;
+#pragma unroll
+  for (int t = 0; t < HD / 32; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {  // registers 4 j .. 4 j + 3 are features 32 t + 8 j + 4 half + (0..3)
+      s16x4 w;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] = bf16_bits(acc[t][4 * j + i] * inv);
+      *reinterpret_cast<s16x4*>(o + 32 * t + 8 * j + 4 * half) = w;
+    }
+}
+
+// tiles[t] = (table row of the sequence, first flat token, number of tokens <= 128)
+extern "C" int pae_attn_prefill_long_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                          const void* k_cache, const void* v_cache, const int* tiles,
+                                          int num_tiles, const int* positions, const int* block_tables,
+                                          int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
+                                          hipStream_t stream) {
+  if (int rc = check_common("attn_prefill_long", nh, nkv, hd, bs, max_blocks, window)) return rc;
+  PAE_REQUIRE(nh <= 65535, "attn_prefill_long: grid too large");
+  if (num_tiles <= 0) return 0;
+  const float scale_log2 = scale * LOG2E;
+  dim3 grid(num_tiles, nh);
+#define CALL(HD)                                                                                            \
+  attn_prefill_lds_kernel<HD, (HD <= 128 ? 64 : 32)><<<grid, 256, 0, stream>>>(                             \
+      (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, \
+      tiles, positions, block_tables, max_blocks, bs, nh, nkv, scale_log2, window)
+  FOR_HEAD_DIM(hd, CALL)
+#undef CALL
+  return pae_check_launch("attn_prefill_long");
+}

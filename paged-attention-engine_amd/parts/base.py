@@ -54,10 +54,12 @@ class StepContext:
     q_lens: List[int] = field(default_factory=list)     # rows of each sequence in this step
     past_lens: List[int] = field(default_factory=list)  # tokens each sequence held before the step
     host_slots: List[int] = field(default_factory=list)
-    # work lists of the attention kernels: sequences that bring one token, and runs of
-    # up to 32 consecutive tokens of the others as (table row, first flat token, count)
+    # work lists of the attention kernels: sequences that bring one token; runs of up to 32
+    # consecutive tokens of sequences that bring 2..32, and runs of up to 128 of those that
+    # bring more, each as (table row, first flat token, count)
     decode_tokens: Optional[torch.Tensor] = None   # int32 [number of single-token sequences]
-    prefill_tiles: Optional[torch.Tensor] = None   # int32 [number of runs, 3]
+    prefill_tiles: Optional[torch.Tensor] = None   # int32 [number of short runs, 3]
+    prefill_long_tiles: Optional[torch.Tensor] = None  # int32 [number of long runs, 3]
     # set by the model for the stop that is running
     entry: int = 0                     # index in the schedule
     cache_entry: int = 0               # the stop whose cache is read (entry itself unless it borrows)

@@ -281,11 +281,17 @@ def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=
     else:
         starts = [sum(q_lens[:s]) for s in range(len(q_lens))]
         dec = [starts[s] for s in range(len(q_lens)) if q_lens[s] == 1]
-        tiles = []
+        tiles, long_tiles = [], []
         for s, ql in enumerate(q_lens):
-            if ql > 1:
+            if ql > 32 and kind != "mfma_short":
+                for first in range(0, ql, 128):
+                    long_tiles.append([s, starts[s] + first, min(128, ql - first)])
+            elif ql > 1:
                 for first in range(0, ql, 32):
                     tiles.append([s, starts[s] + first, min(32, ql - first)])
+        if long_tiles:
+            K().attn_prefill(out, qd, d(kp), d(vp), d(long_tiles, torch.int32), pos_d, tab_d, nh, nkv, hd, scale,
+                             window, long=True)
         if dec:
             K().attn_decode(out, qd, d(kp), d(vp), d(dec, torch.int32), pos_d, seq_d, tab_d, nh, nkv, hd, scale, window)
         if tiles:
@@ -331,10 +337,18 @@ def test_one_far_key_stands_out(kind, key_pos, window, seen):
         assert want[0].abs().max() > 0.5
 
 
-@pytest.mark.parametrize("q_len", [2, 31, 32, 33, 64, 100])
-def test_matrix_core_prefill_from_empty_and_warm(q_len):
-    got, want = run_attention("mfma", "bfloat16", 12, 2, 128, 16, 0, [q_len, 200 + q_len], [q_len, q_len])
+@pytest.mark.parametrize("kind", ["mfma", "mfma_short"])
+@pytest.mark.parametrize("q_len", [2, 31, 32, 33, 64, 100, 128, 129, 300])
+def test_matrix_core_prefill_from_empty_and_warm(kind, q_len):
+    got, want = run_attention(kind, "bfloat16", 12, 2, 128, 16, 0, [q_len, 200 + q_len], [q_len, q_len])
     assert (got - want).abs().max() <= 3e-2
+
+
+@pytest.mark.parametrize("nh,nkv,hd,bs,window", MFMA_SHAPES)
+def test_matrix_core_long_prefill_shapes(nh, nkv, hd, bs, window):
+    got, want = run_attention("mfma", "bfloat16", nh, nkv, hd, bs, window, [333, 700, 130], [333, 190, 77])
+    err = (got - want).abs().max(dim=1).values
+    assert float(err.max()) <= 3e-2, f"worst rows: {torch.topk(err, 5)}"
 
 
 # ------------------------------------------------------------------ sampling
