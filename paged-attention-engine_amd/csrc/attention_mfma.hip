@@ -406,7 +406,7 @@ extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* 
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 template <int HD, int BN>
-__global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
+__global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_lds_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ tiles,
     const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int bs, int nh,
@@ -430,6 +430,9 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
   const int start = (live && window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int wave_hi = min(pos0 + wave * 32 + 31, pos0 + ntok - 1);  // last position of this wavefront
   const bool wave_live = wave * 32 < ntok;
+  const bool wave_full = wave * 32 + 32 <= ntok;  // no dead column in this wavefront
+  const int wave_lo = pos0 + wave * 32;            // its first position, and the window start of its last
+  const int wave_start = (window > 0 && wave_hi - window + 1 > 0) ? wave_hi - window + 1 : 0;
   const int lo = (window > 0 && pos0 - window + 1 > 0) ? (pos0 - window + 1) / BN * BN : 0;
   const int hi = pos0 + ntok - 1;
 
@@ -455,7 +458,8 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
     for (int p = 0; p < PAGES; ++p) {
       const int key = key0 + 16 * p;
       const int kc = key <= hi ? key : key0;  // pages past the end repeat the first one (never used)
-      const int64_t base = ((int64_t)table[kc / bs] * nkv + kvh) * page_elems;
+      // a page the window has passed was given back (its entry is -1): every key of it is masked, read page 0
+      const int64_t base = ((int64_t)max(table[kc / bs], 0) * nkv + kvh) * page_elems;
       const bf16_t* kp = k_cache + base + (int64_t)(kc % bs) * HD;  // [16 keys][HD], contiguous
       const bf16_t* vp = v_cache + base + kc % bs;                  // [HD][bs]: 16 keys of each feature
 #pragma unroll
@@ -491,53 +495,75 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
     __syncthreads();
     if (key0 + BN <= hi) fetch(key0 + BN);
     if (!wave_live || key0 > wave_hi) continue;  // nothing for this wavefront in the tile (causal)
+    // scores of the whole tile first, then one softmax update and one rescale for it
+    f32x16 s[BN / 32];
 #pragma unroll
     for (int kb = 0; kb < BN / 32; ++kb) {
-      f32x16 s;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) s[v] = 0.f;
+      for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+      bf16x8 kf[HD / 16];  // all key fragments of the block are read before the first product uses one
 #pragma unroll
-      for (int ks = 0; ks < HD / 16; ++ks) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(k_lds + (32 * kb + col) * KS + 16 * ks + 8 * half);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s, 0, 0, 0);
-      }
-      float mx = NEG_BIG;
+      for (int ks = 0; ks < HD / 16; ++ks)
+        kf[ks] = *reinterpret_cast<const bf16x8*>(k_lds + (32 * kb + col) * KS + 16 * ks + 8 * half);
+#pragma unroll
+      for (int ks = 0; ks < HD / 16; ++ks) s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], s[kb], 0, 0, 0);
+    }
+    // a tile that every token of this wavefront sees whole needs no mask
+    const bool whole = wave_full && key0 + BN - 1 <= wave_lo && key0 >= wave_start;
+    float mx = NEG_BIG;
+    if (whole) {
+#pragma unroll
+      for (int kb = 0; kb < BN / 32; ++kb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          s[kb][v] *= scale_log2;
+          mx = fmaxf(mx, s[kb][v]);
+        }
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < BN / 32; ++kb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int key = key0 + 32 * kb + 8 * (v / 4) + 4 * half + v % 4;
+          s[kb][v] = (key <= pos && key >= start) ? s[kb][v] * scale_log2 : -INFINITY;
+          mx = fmaxf(mx, s[kb][v]);
+        }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, PAE_WAVE));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = exp2f(m - m_new);
+    m = m_new;
+    float psum = 0.f;
+    bf16x8 pb[BN / 32][2];
+#pragma unroll
+    for (int kb = 0; kb < BN / 32; ++kb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int key = key0 + 32 * kb + 8 * (v / 4) + 4 * half + v % 4;
-        s[v] = (key <= pos && key >= start) ? s[v] * scale_log2 : -INFINITY;
-        mx = fmaxf(mx, s[v]);
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, PAE_WAVE));
-      const float m_new = fmaxf(m, mx);
-      const float alpha = exp2f(m - m_new);
-      m = m_new;
-      float psum = 0.f;
-      bf16x8 pb[2];
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float p = exp2f(s[v] - m_new);
+        const float p = exp2f(s[kb][v] - m_new);
         psum += p;
-        pb[v / 8][v % 8] = (__bf16)p;
+        pb[kb][v / 8][v % 8] = (__bf16)p;
       }
-      l = l * alpha + psum;
+    l = l * alpha + psum;
 #pragma unroll
-      for (int t = 0; t < HD / 32; ++t) {
+    for (int t = 0; t < HD / 32; ++t) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[t][v] *= alpha;
+      for (int v = 0; v < 16; ++v) acc[t][v] *= alpha;
+      // value fragments: keys 16 st + 4 half + (0..3) and 16 st + 8 + 4 half + (0..3) of block kb, feature 32 t + col
+      bf16x8 vf[BN / 32][2];
+#pragma unroll
+      for (int kb = 0; kb < BN / 32; ++kb)
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
-          // values of keys 16 st + 4 half + (0..3) and 16 st + 8 + 4 half + (0..3) of this block, feature 32 t + col
           const bf16_t* vrow = v_lds + (32 * t + col) * VS + 32 * kb + 16 * st + 4 * half;
-          bf16x8 vf;
-          const s16x4 a = *reinterpret_cast<const s16x4*>(vrow);
-          const s16x4 b = *reinterpret_cast<const s16x4*>(vrow + 8);
-          s16x4* dst = reinterpret_cast<s16x4*>(&vf);
-          dst[0] = a;
-          dst[1] = b;
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[st], acc[t], 0, 0, 0);
+          s16x4* dst = reinterpret_cast<s16x4*>(&vf[kb][st]);
+          dst[0] = *reinterpret_cast<const s16x4*>(vrow);
+          dst[1] = *reinterpret_cast<const s16x4*>(vrow + 8);
         }
-      }
+#pragma unroll
+      for (int kb = 0; kb < BN / 32; ++kb)
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[kb][st], pb[kb][st], acc[t], 0, 0, 0);
     }
   }
   l += __shfl_xor(l, 32, PAE_WAVE);

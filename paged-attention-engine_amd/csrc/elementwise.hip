@@ -322,6 +322,33 @@ __global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ x, int 
   out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
 }
 
+// Eight bfloat16 outputs per thread (16-byte loads and stores): used when the width and
+// the block size are multiples of 8.
+__global__ void swiglu_vec8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ x, int inter, int block,
+                                   int64_t total_vecs) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total_vecs) return;
+  const int per_row = inter / 8;
+  const int64_t t = idx / per_row;
+  const int j = (int)(idx % per_row) * 8;
+  const int64_t gi = block ? (int64_t)(j / block) * 2 * block + j % block : j;
+  const int64_t ui = block ? gi + block : (int64_t)inter + j;
+  const uint4 g4 = *reinterpret_cast<const uint4*>(x + t * 2 * inter + gi);
+  const uint4 u4 = *reinterpret_cast<const uint4*>(x + t * 2 * inter + ui);
+  const unsigned gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+  unsigned ow[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
+    const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
+    const bf16_t o0 = __float2bfloat16(g0 / (1.0f + expf(-g0)) * u0);
+    const bf16_t o1 = __float2bfloat16(g1 / (1.0f + expf(-g1)) * u1);
+    ow[k] = (unsigned)(*reinterpret_cast<const unsigned short*>(&o0)) |
+            ((unsigned)(*reinterpret_cast<const unsigned short*>(&o1)) << 16);
+  }
+  *reinterpret_cast<uint4*>(out + t * inter + j) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 extern "C" int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, int block,
                           hipStream_t stream) {
   PAE_REQUIRE(num_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", num_tokens, inter);
@@ -331,9 +358,13 @@ extern "C" int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, i
   const unsigned blocks = (unsigned)((total + 255) / 256);
   if (dtype == PAE_F32)
     swiglu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)x, inter, block, total);
-  else if (dtype == PAE_BF16)
-    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, inter, block, total);
-  else
+  else if (dtype == PAE_BF16) {
+    if (inter % 8 == 0 && block % 8 == 0)
+      swiglu_vec8_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x,
+                                                                                 inter, block, total / 8);
+    else
+      swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, inter, block, total);
+  } else
     return pae_fail("swiglu: unknown dtype code %d", dtype);
   return pae_check_launch("swiglu");
 }
