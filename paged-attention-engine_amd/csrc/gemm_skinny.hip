@@ -30,13 +30,16 @@ __device__ __forceinline__ short to_bf16_bits(float x) {
   return *reinterpret_cast<const short*>(&h);
 }
 
-template <int MT, int EPI>
+// MT: column tiles of 16 rows of A; RT: tiles of 16 weight rows per workgroup.  With more
+// rows of A a workgroup takes more weight rows, so that the activations, which every
+// workgroup re-reads from L2, do not outweigh the weights.
+template <int MT, int RT, int EPI>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out, int64_t ldc,
                                                           const bf16_t* __restrict__ A, int64_t lda,
                                                           const bf16_t* __restrict__ W,
                                                           const void* __restrict__ bias, int b_is_f32, int M,
                                                           int N, int K, int k_per_split, int64_t part_stride) {
-  constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
+  static_assert(EPI != EPI_SWIGLU || RT % 2 == 0, "the gated epilogue pairs a gate tile with its up tile");
   __shared__ float s_part[3][RT * MT * 4][PAE_WAVE];
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
@@ -116,41 +119,48 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
         for (int i = 0; i < 4; ++i) acc[rt][mt][i] += s_part[w][(rt * MT + mt) * 4 + i][lane];
 
   const bool vec = ldc % 4 == 0;  // rows of out keep 8- and 16-byte stores aligned
-  // lane holds, per column tile mt, row m = 16 mt + r of A and weight rows 4 g4 + i of the tile
+  // lane holds, per column tile mt, row m = 16 mt + r of A and weight rows 4 g4 + i of each row tile
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + r;
     if (m >= M) continue;
     if (EPI == EPI_SWIGLU) {
-      const int j = blockIdx.x * 16 + 4 * g4;  // output feature of register 0
-      if (j >= N / 2) continue;                // N counts gate and up rows; whole blocks of 16 only
-      s16x4 v;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float g = acc[0][mt][i], u = acc[1][mt][i];
-        v[i] = to_bf16_bits(g / (1.0f + expf(-g)) * u);
+      for (int pair = 0; pair < RT / 2; ++pair) {  // tiles 2 pair (gate) and 2 pair + 1 (up)
+        const int j = (blockIdx.x * (RT / 2) + pair) * 16 + 4 * g4;  // output feature of register 0
+        if (j >= N / 2) continue;                                    // N counts gate and up rows
+        s16x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float g = acc[2 * pair][mt][i], u = acc[2 * pair + 1][mt][i];
+          v[i] = to_bf16_bits(g / (1.0f + expf(-g)) * u);
+        }
+        *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j) = v;
       }
-      *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j) = v;
     } else {
-      const int n = n0 + 4 * g4;
-      if (n >= N) continue;
-      float v[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = acc[0][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f);
-      if (EPI == EPI_F32) {
-        float* dst = (float*)out + (int64_t)blockIdx.y * part_stride + (int64_t)m * ldc + n;
-        if (vec && n + 4 <= N) *reinterpret_cast<f32x4*>(dst) = (f32x4){v[0], v[1], v[2], v[3]};
-        else
-          for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = v[i];
-      } else {
-        bf16_t* dst = (bf16_t*)out + (int64_t)m * ldc + n;
-        if (vec && n + 4 <= N) {
-          s16x4 p;
+      for (int rt = 0; rt < RT; ++rt) {
+        const int n = n0 + 16 * rt + 4 * g4;
+        if (n >= N) continue;
+        float v[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) p[i] = to_bf16_bits(v[i]);
-          *reinterpret_cast<s16x4*>(dst) = p;
-        } else
-          for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = __float2bfloat16(v[i]);
+        for (int i = 0; i < 4; ++i)
+          v[i] = acc[rt][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f);
+        if (EPI == EPI_F32) {
+          float* dst = (float*)out + (int64_t)blockIdx.y * part_stride + (int64_t)m * ldc + n;
+          if (vec && n + 4 <= N) *reinterpret_cast<f32x4*>(dst) = (f32x4){v[0], v[1], v[2], v[3]};
+          else
+            for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = v[i];
+        } else {
+          bf16_t* dst = (bf16_t*)out + (int64_t)m * ldc + n;
+          if (vec && n + 4 <= N) {
+            s16x4 p;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p[i] = to_bf16_bits(v[i]);
+            *reinterpret_cast<s16x4*>(dst) = p;
+          } else
+            for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = __float2bfloat16(v[i]);
+        }
       }
     }
   }
@@ -169,21 +179,22 @@ extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void*
   PAE_REQUIRE(!(bias && splits > 1), "gemm_skinny: a bias cannot be combined with partial sums");
   PAE_REQUIRE(epilogue != EPI_SWIGLU || (N % 32 == 0 && ldc % 4 == 0), "gemm_skinny: gated epilogue needs N %% 32 == 0, got %d", N);
   if (M == 0) return 0;
-  const int rows_per_wg = epilogue == EPI_SWIGLU ? 32 : 16;
+  // weight rows per workgroup: 16 for up to 16 rows of A, else 32 (see the kernel)
+  const int mt = (M + 15) / 16;
+  const int rt = (mt >= 2 || epilogue == EPI_SWIGLU) ? 2 : 1;
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + 127) / 128 * 128;
   PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "gemm_skinny: %d k ranges are too many for K=%d", splits, K);
-  dim3 grid((N + rows_per_wg - 1) / rows_per_wg, splits);
-  const int mt = (M + 15) / 16;
-#define LAUNCH(MT, EPI)                                                                                       \
-  gemm_skinny_kernel<MT, EPI><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, bias, \
-                                                        b_is_f32, M, N, K, k_per_split, part_stride)
-#define BY_MT(EPI)                       \
-  switch (mt) {                          \
-    case 1: LAUNCH(1, EPI); break;       \
-    case 2: LAUNCH(2, EPI); break;       \
-    case 3: LAUNCH(3, EPI); break;       \
-    default: LAUNCH(4, EPI); break;      \
+  dim3 grid((N + 16 * rt - 1) / (16 * rt), splits);
+#define LAUNCH(MT, RT, EPI)                                                                                   \
+  gemm_skinny_kernel<MT, RT, EPI><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
+                                                            bias, b_is_f32, M, N, K, k_per_split, part_stride)
+#define BY_MT(EPI)                                                   \
+  switch (mt) {                                                      \
+    case 1: LAUNCH(1, (EPI == EPI_SWIGLU ? 2 : 1), EPI); break;       \
+    case 2: LAUNCH(2, 2, EPI); break;                                \
+    case 3: LAUNCH(3, 2, EPI); break;                                \
+    default: LAUNCH(4, 2, EPI); break;                               \
   }
   switch (epilogue) {
     case EPI_BF16: BY_MT(EPI_BF16); break;

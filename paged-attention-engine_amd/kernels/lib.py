@@ -213,9 +213,11 @@ def skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0 and a.stride(1) == 1)
 
 
-def skinny_splits(N: int, K: int) -> int:
-    """k ranges for a product whose consumer adds float32 partials: enough workgroups to fill the chip."""
-    tiles = -(-N // 16)
+def skinny_splits(N: int, K: int, M: int = 1) -> int:
+    """k ranges for a product whose consumer adds float32 partials: enough workgroups to fill the
+    chip (a workgroup takes 16 weight rows, or 32 with more than 16 rows of activations)."""
+    rows = 32 if M > 16 else 16
+    tiles = -(-N // rows)
     wanted = max(1, min(512 // tiles, K // 256, 8))
     k_per = -(-(-(-K // wanted)) // 128) * 128
     return -(-K // k_per)

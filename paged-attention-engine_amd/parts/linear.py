@@ -55,7 +55,7 @@ class Linear:
         """The product as a residual branch's output: [M, N] in x's dtype, or float32
         partial sums [P, M, N] that the next norm adds up in order (no bias then)."""
         if x.dtype == torch.bfloat16 and self.bias is None and x.shape[0] and K.skinny_supported(x, self.weight):
-            splits = K.skinny_splits(self.out_features, self.in_features)
+            splits = K.skinny_splits(self.out_features, self.in_features, x.shape[0])
             out = torch.empty((splits, x.shape[0], self.out_features), dtype=torch.float32, device=x.device)
             K.gemm_skinny(out, x, self.weight, None, K.EPI_F32, splits)
             return out
