@@ -87,16 +87,42 @@ __device__ __forceinline__ void attn_tile(AttnState<HD, CT>& st, const bf16x8 (&
   }
 }
 
+// Loads are made with the lane order (row = lane / 4, group = lane % 4), so that the four lanes of
+// a quad read contiguous bytes (64 of a key row, 32 of a value row) and the memory pipeline sees
+// one access for them; `kv_to_mfma_order` then moves every register to the order the matrix
+// instruction wants (row = lane % 16, group = lane / 16) with one cross-lane permute each.
 template <int HD>
 __device__ __forceinline__ void load_kv_tile(bf16x8 (&kf)[HD / 32], s16x4 (&vf)[HD / 16], const bf16_t* kp,
                                              const bf16_t* vp, int vstride) {
   const int lane = threadIdx.x % PAE_WAVE;
-  const int r = lane % 16, g4 = lane / 16;
+  const int r = lane / 4, g = lane % 4;
 #pragma unroll
-  for (int j = 0; j < HD / 32; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(kp + r * HD + 32 * j + 8 * g4);
+  for (int j = 0; j < HD / 32; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(kp + r * HD + 32 * j + 8 * g);
 #pragma unroll
   for (int t = 0; t < HD / 16; ++t)
-    vf[t] = *reinterpret_cast<const s16x4*>(vp + (int64_t)(16 * t + r) * vstride + 4 * g4);
+    vf[t] = *reinterpret_cast<const s16x4*>(vp + (int64_t)(16 * t + r) * vstride + 4 * g);
+}
+
+template <int HD>
+__device__ __forceinline__ void kv_to_mfma_order(bf16x8 (&kf)[HD / 32], s16x4 (&vf)[HD / 16]) {
+  typedef __attribute__((ext_vector_type(4))) int i32x4;
+  typedef __attribute__((ext_vector_type(2))) int i32x2;
+  const int lane = threadIdx.x % PAE_WAVE;
+  const int fetch_from = ((lane % 16) * 4 + lane / 16) * 4;  // byte address of the source lane
+#pragma unroll
+  for (int j = 0; j < HD / 32; ++j) {
+    i32x4 raw = *reinterpret_cast<i32x4*>(&kf[j]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = __builtin_amdgcn_ds_bpermute(fetch_from, raw[i]);
+    kf[j] = *reinterpret_cast<bf16x8*>(&raw);
+  }
+#pragma unroll
+  for (int t = 0; t < HD / 16; ++t) {
+    i32x2 raw = *reinterpret_cast<i32x2*>(&vf[t]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) raw[i] = __builtin_amdgcn_ds_bpermute(fetch_from, raw[i]);
+    vf[t] = *reinterpret_cast<s16x4*>(&raw);
+  }
 }
 
 // ------------------------------------------------------------------ decode
@@ -161,6 +187,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
   for (int j = 0; j < TPW; ++j) {
     const int tile = tile_lo + wave + 4 * j;
+    kv_to_mfma_order<HD>(kf[j], vf[j]);  // in every lane of the wavefront, used or not
     if (tile < tile_hi) attn_tile<HD, 1>(st, kf[j], vf[j], qf, tile * 16, pos, start, scale_log2);
   }
 
@@ -299,6 +326,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const int blk = table[key0 / bs];
     const int64_t base = ((int64_t)blk * nkv + kvh) * page_elems;
     load_kv_tile<HD>(kf, vf, k_cache + base + (int64_t)(key0 % bs) * HD, v_cache + base + key0 % bs, bs);
+    kv_to_mfma_order<HD>(kf, vf);
     attn_tile<HD, PREFILL_CT>(st, kf, vf, qf, key0, pos, start, scale_log2);
   }
 #pragma unroll

@@ -23,17 +23,26 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 #define EPI_BF16 0
 #define EPI_F32 1
 #define EPI_SWIGLU 2
-#define SKINNY_U 4  // k steps of a wavefront whose loads are in flight together
+
+// A fragment loaded as (row = lane / 4, k group = lane % 4) moved to (row = lane % 16, k group = lane / 16).
+__device__ __forceinline__ bf16x8 to_mfma_order(bf16x8 v, int fetch_from) {
+  typedef __attribute__((ext_vector_type(4))) int i32x4;
+  i32x4 raw = *reinterpret_cast<i32x4*>(&v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) raw[i] = __builtin_amdgcn_ds_bpermute(fetch_from, raw[i]);
+  return *reinterpret_cast<bf16x8*>(&raw);
+}
 
 __device__ __forceinline__ short to_bf16_bits(float x) {
   const bf16_t h = __float2bfloat16(x);
   return *reinterpret_cast<const short*>(&h);
 }
 
-// MT: column tiles of 16 rows of A; RT: tiles of 16 weight rows per workgroup.  With more
+// MT: column tiles of 16 rows of A; RT: tiles of 16 weight rows per workgroup; SKINNY_U: k steps
+// of a wavefront whose loads are in flight together.  With more
 // rows of A a workgroup takes more weight rows, so that the activations, which every
 // workgroup re-reads from L2, do not outweigh the weights.
-template <int MT, int RT, int EPI>
+template <int MT, int RT, int EPI, int SKINNY_U>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out, int64_t ldc,
                                                           const bf16_t* __restrict__ A, int64_t lda,
                                                           const bf16_t* __restrict__ W,
@@ -47,21 +56,23 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
   const int k_lo = blockIdx.y * k_per_split;
   const int k_hi = min(K, k_lo + k_per_split);
 
+  // Loads are made with the lane order (row = lane / 4, k group = lane % 4): the four lanes of a
+  // quad then read 64 contiguous bytes, which the memory pipeline handles as one access.  The
+  // matrix instruction wants (row = lane % 16, k group = lane / 16); one cross-lane permute per
+  // register moves a loaded fragment into that order.
+  const int lrow = lane / 4, lkg = lane % 4;
+  const int fetch_from = ((lane % 16) * 4 + lane / 16) * 4;  // byte address of the source lane for ds_bpermute
   const bf16_t* wrow[RT];
-  bool wok[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int n = n0 + 16 * rt + r;
-    wok[rt] = n < N;
-    wrow[rt] = W + (int64_t)(wok[rt] ? n : N - 1) * K;
+    const int n = n0 + 16 * rt + lrow;
+    wrow[rt] = W + (int64_t)(n < N ? n : N - 1) * K;  // rows past N are loaded from the last row and never stored
   }
   const bf16_t* arow[MT];
-  bool aok[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int m = 16 * mt + r;
-    aok[mt] = m < M;
-    arow[mt] = A + (int64_t)(aok[mt] ? m : 0) * lda;
+    const int m = 16 * mt + lrow;
+    arow[mt] = A + (int64_t)(m < M ? m : M - 1) * lda;
   }
   f32x4 acc[RT][MT];
 #pragma unroll
@@ -76,11 +87,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
   const bf16x8 zero = {};
   for (int kb = k_lo + 32 * wave; kb < k_hi; kb += 128 * SKINNY_U) {
     bf16x8 wf[SKINNY_U][RT], af[SKINNY_U][MT];
-    bool kok[SKINNY_U];
 #pragma unroll
     for (int u = 0; u < SKINNY_U; ++u) {
-      const int k = kb + 128 * u + 8 * g4;
-      kok[u] = k < k_hi;  // K and the range bounds are multiples of 8: all 8 elements in or out
+      const int k = kb + 128 * u + 8 * lkg;
       const int kc = k < K - 8 ? k : K - 8;
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) wf[u][rt] = *reinterpret_cast<const bf16x8*>(wrow[rt] + kc);
@@ -89,9 +98,15 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
     }
 #pragma unroll
     for (int u = 0; u < SKINNY_U; ++u) {
+      // K and the range bounds are multiples of 8: a lane's 8 elements are all in or all out
+      const bool kok = kb + 128 * u + 8 * g4 < k_hi;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) af[u][mt] = to_mfma_order(af[u][mt], fetch_from);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
-        const bf16x8 w = kok[u] ? wf[u][rt] : zero;
+        // the permute runs in every lane (a lane that skipped it could not be read by the others)
+        const bf16x8 moved = to_mfma_order(wf[u][rt], fetch_from);
+        const bf16x8 w = kok ? moved : zero;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
           acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, af[u][mt], acc[rt][mt], 0, 0, 0);
@@ -186,9 +201,10 @@ extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void*
   k_per_split = (k_per_split + 127) / 128 * 128;
   PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "gemm_skinny: %d k ranges are too many for K=%d", splits, K);
   dim3 grid((N + 16 * rt - 1) / (16 * rt), splits);
-#define LAUNCH(MT, RT, EPI)                                                                                   \
-  gemm_skinny_kernel<MT, RT, EPI><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
-                                                            bias, b_is_f32, M, N, K, k_per_split, part_stride)
+  // four k steps of loads in flight per wavefront: deeper prefetch costs registers and measured slower
+#define LAUNCH(MT, RT, EPI)                                                                                  \
+  gemm_skinny_kernel<MT, RT, EPI, 4><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
+                                                               bias, b_is_f32, M, N, K, k_per_split, part_stride)
 #define BY_MT(EPI)                                                   \
   switch (mt) {                                                      \
     case 1: LAUNCH(1, (EPI == EPI_SWIGLU ? 2 : 1), EPI); break;       \
