@@ -24,6 +24,10 @@ int pae_gemm_plain(int in_dtype, int out_dtype, void* C, int64_t ldc, const void
 int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
                     const void* bias, int b_is_f32, int M, int N, int K, int splits, int64_t part_stride,
                     hipStream_t stream);
+int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int64_t lda, const void* W, const void* bias,
+                         int b_is_f32, int M, int K, int nh, int nkv, int hd, int rot, const float* inv_freq,
+                         const int* positions, const int* tok_seq, const int* block_tables, int max_blocks, int bs,
+                         void* k_cache, void* v_cache, hipStream_t stream);
 int pae_paged_attention_generic(int dtype, void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                 const void* k_cache, const void* v_cache, const int* positions,
                                 const int* tok_seq, const int* block_tables, int max_blocks, int bs,

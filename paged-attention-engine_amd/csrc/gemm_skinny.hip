@@ -12,7 +12,12 @@
 //
 // Epilogues: bfloat16 out with bias; float32 out (logits, or partial sums);
 // SiLU gate: rows come in blocks of 16 gate rows followed by their 16 up rows,
-// and out[m, j] = silu(gate_j) * up_j (engine/model.py:317-320 of the reference).
+// and out[m, j] = silu(gate_j) * up_j (engine/model.py:317-320 of the reference);
+// rotation: W holds the query, key and value projections of an attention layer, a
+// tile takes 8 features of a head and the 8 they are rotated with, queries come out
+// rotated and keys and values go straight to their cache slots (engine/model.py:
+// 155-161, engine/attention.py:374-385,409-410), so the projection's result never
+// makes a round trip through memory.
 #include "common.h"
 #include "api.h"
 
@@ -23,6 +28,26 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 #define EPI_BF16 0
 #define EPI_F32 1
 #define EPI_SWIGLU 2
+#define EPI_ROPE 3
+
+// What the rotating epilogue needs beside the product: the head geometry, the
+// rotation's frequencies, every row's position and sequence, and the paged cache.
+struct SkinnyRope {
+  const float* inv_freq;    // [rot / 2], or null without rotation
+  const int* positions;     // [M]
+  const int* tok_seq;       // [M] row of block_tables
+  const int* block_tables;  // [sequences][max_blocks]
+  bf16_t* k_cache;          // [block][kv head][bs][hd]
+  bf16_t* v_cache;          // [block][kv head][hd][bs]
+  int nh, nkv, hd, rot, max_blocks, bs;
+};
+
+// Feature within its head of row `r` of the `j`-th tile of a head: a tile inside the rotated
+// part holds features 8 j .. 8 j + 7 (rows 0-7) and their partners rot / 2 + 8 j .. (rows 8-15);
+// tiles past it hold 16 consecutive features that pass through.
+__device__ __forceinline__ int rope_feature(int j, int r, int rot) {
+  return 16 * j < rot ? (r < 8 ? 8 * j + r : rot / 2 + 8 * j + r - 8) : 16 * j + r;
+}
 
 // A fragment loaded as (row = lane / 4, k group = lane % 4) moved to (row = lane % 16, k group = lane / 16).
 __device__ __forceinline__ bf16x8 to_mfma_order(bf16x8 v, int fetch_from) {
@@ -47,7 +72,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
                                                           const bf16_t* __restrict__ A, int64_t lda,
                                                           const bf16_t* __restrict__ W,
                                                           const void* __restrict__ bias, int b_is_f32, int M,
-                                                          int N, int K, int k_per_split, int64_t part_stride) {
+                                                          int N, int K, int k_per_split, int64_t part_stride,
+                                                          SkinnyRope rope) {
   static_assert(EPI != EPI_SWIGLU || RT % 2 == 0, "the gated epilogue pairs a gate tile with its up tile");
   __shared__ float s_part[3][RT * MT * 4][PAE_WAVE];
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
@@ -65,7 +91,11 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
   const bf16_t* wrow[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int n = n0 + 16 * rt + lrow;
+    int n = n0 + 16 * rt + lrow;
+    if (EPI == EPI_ROPE) {
+      const int tile = blockIdx.x * RT + rt, per_head = rope.hd / 16;
+      n = tile / per_head * rope.hd + rope_feature(tile % per_head, lrow, rope.rot);
+    }
     wrow[rt] = W + (int64_t)(n < N ? n : N - 1) * K;  // rows past N are loaded from the last row and never stored
   }
   const bf16_t* arow[MT];
@@ -133,6 +163,59 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[rt][mt][i] += s_part[w][(rt * MT + mt) * 4 + i][lane];
 
+  if (EPI == EPI_ROPE) {
+    // lane holds row m = 16 mt + r of A and rows 4 g4 + i of each tile: lanes 0-31 the lower
+    // features of the pairs, lanes 32-63 (same m) their partners
+    const int per_head = rope.hd / 16;
+    const int64_t head_step = (int64_t)rope.bs * rope.hd;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = 16 * mt + r;
+      const int mc = m < M ? m : M - 1;
+      const int pos = rope.positions[mc];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int tile = blockIdx.x * RT + rt;
+        const int head = tile / per_head, j = tile % per_head;
+        const bool rotated = 16 * j < rope.rot && head < rope.nh + rope.nkv;  // values keep the tile layout, unrotated
+        const int f0 = rope_feature(j, 4 * g4, rope.rot);  // first of this lane's 4 consecutive features
+        const int n = head * rope.hd + f0;
+        s16x4 res;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          // the projection is rounded to bfloat16 before the rotation, as where the two are separate kernels
+          const float own = __bfloat162float(__float2bfloat16(
+              acc[rt][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f)));
+          const float other = __shfl_xor(own, 32);  // in every lane
+          float o = own;
+          if (rotated) {
+            float sn, cs;
+            sincosf((float)pos * rope.inv_freq[8 * j + (4 * g4 + i) % 8], &sn, &cs);
+            o = g4 < 2 ? own * cs - other * sn : own * cs + other * sn;
+          }
+          res[i] = to_bf16_bits(o);
+        }
+        if (m >= M || n >= N) continue;
+        if (head < rope.nh) {
+          *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + n) = res;
+          continue;
+        }
+        const int off = pos % rope.bs;
+        const int64_t page = (int64_t)rope.block_tables[(int64_t)rope.tok_seq[m] * rope.max_blocks + pos / rope.bs] *
+                             rope.nkv * head_step;
+        if (head < rope.nh + rope.nkv) {
+          *reinterpret_cast<s16x4*>(rope.k_cache + page + (head - rope.nh) * head_step + (int64_t)off * rope.hd + f0) = res;
+        } else {
+          short* dst = reinterpret_cast<short*>(rope.v_cache) + page + (head - rope.nh - rope.nkv) * head_step +
+                       (int64_t)f0 * rope.bs + off;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[(int64_t)i * rope.bs] = res[i];
+        }
+      }
+    }
+    return;
+  }
+
   const bool vec = ldc % 4 == 0;  // rows of out keep 8- and 16-byte stores aligned
   // lane holds, per column tile mt, row m = 16 mt + r of A and weight rows 4 g4 + i of each row tile
 #pragma unroll
@@ -184,9 +267,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
 // epilogue: 0 bfloat16 out (+bias), 1 float32 out (`splits` partials of `part_stride`
 // elements each when splits > 1; a bias only with one split), 2 SiLU gate (N counts the
 // interleaved gate and up rows; out is [M, N / 2]).
-extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
-                               const void* bias, int b_is_f32, int M, int N, int K, int splits,
-                               int64_t part_stride, hipStream_t stream) {
+static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
+                         const void* bias, int b_is_f32, int M, int N, int K, int splits, int64_t part_stride,
+                         const SkinnyRope& rope, hipStream_t stream) {
   PAE_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d is outside 0..64", M);
   PAE_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && lda % 8 == 0, "gemm_skinny: N=%d K=%d lda=%lld (K and lda must be multiples of 8)",
               N, K, (long long)lda);
@@ -204,7 +287,7 @@ extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void*
   // four k steps of loads in flight per wavefront: deeper prefetch costs registers and measured slower
 #define LAUNCH(MT, RT, EPI)                                                                                  \
   gemm_skinny_kernel<MT, RT, EPI, 4><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
-                                                               bias, b_is_f32, M, N, K, k_per_split, part_stride)
+                                                               bias, b_is_f32, M, N, K, k_per_split, part_stride, rope)
 #define BY_MT(EPI)                                                   \
   switch (mt) {                                                      \
     case 1: LAUNCH(1, (EPI == EPI_SWIGLU ? 2 : 1), EPI); break;       \
@@ -216,9 +299,39 @@ extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void*
     case EPI_BF16: BY_MT(EPI_BF16); break;
     case EPI_F32: BY_MT(EPI_F32); break;
     case EPI_SWIGLU: BY_MT(EPI_SWIGLU); break;
+    case EPI_ROPE: BY_MT(EPI_ROPE); break;
     default: return pae_fail("gemm_skinny: unknown epilogue %d", epilogue);
   }
 #undef BY_MT
 #undef LAUNCH
   return pae_check_launch("gemm_skinny");
+}
+
+extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
+                               const void* bias, int b_is_f32, int M, int N, int K, int splits,
+                               int64_t part_stride, hipStream_t stream) {
+  PAE_REQUIRE(epilogue != EPI_ROPE, "gemm_skinny: the rotating epilogue has an entry point of its own");
+  return launch_skinny(epilogue, out, ldc, A, lda, W, bias, b_is_f32, M, N, K, splits, part_stride, SkinnyRope{},
+                       stream);
+}
+
+// q_out[M, nh * hd] = rotated queries of A * W^T (+ bias), W = [(nh + 2 nkv) * hd, K] holding the
+// query, key and value projections in that order; rotated keys and raw values of every row go to
+// slot block_tables[tok_seq[m]][positions[m] / bs] * bs + positions[m] % bs of the cache.  With
+// nkv == 0 only queries are projected and nothing is stored.  rot == 0 (inv_freq null) rotates nothing.
+extern "C" int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int64_t lda, const void* W,
+                                    const void* bias, int b_is_f32, int M, int K, int nh, int nkv, int hd, int rot,
+                                    const float* inv_freq, const int* positions, const int* tok_seq,
+                                    const int* block_tables, int max_blocks, int bs, void* k_cache, void* v_cache,
+                                    hipStream_t stream) {
+  PAE_REQUIRE(nh > 0 && nkv >= 0 && hd > 0 && hd % 16 == 0, "gemm_skinny_rope: bad head sizes nh=%d nkv=%d hd=%d", nh, nkv, hd);
+  PAE_REQUIRE(rot >= 0 && rot <= hd && rot % 16 == 0 && (rot == 0 || inv_freq),
+              "gemm_skinny_rope: rotary_dim %d must be a multiple of 16 up to head_dim %d", rot, hd);
+  PAE_REQUIRE(ldq >= (int64_t)nh * hd && ldq % 4 == 0, "gemm_skinny_rope: row stride %lld of the queries", (long long)ldq);
+  PAE_REQUIRE(positions, "gemm_skinny_rope: positions are missing");
+  PAE_REQUIRE(nkv == 0 || (bs > 0 && max_blocks > 0 && k_cache && v_cache && block_tables && tok_seq),
+              "gemm_skinny_rope: the cache write needs tables and pools");
+  SkinnyRope rope{inv_freq, positions, tok_seq, block_tables, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                  nh, nkv, hd, rot, max_blocks, bs};
+  return launch_skinny(EPI_ROPE, q_out, ldq, A, lda, W, bias, b_is_f32, M, (nh + 2 * nkv) * hd, K, 1, 0, rope, stream);
 }

@@ -57,6 +57,7 @@ def _declare(lib) -> None:
         "pae_rope_kv_write": [I, P, L, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P],
         "pae_swiglu": [I, P, P, I, I, I, P],
         "pae_gemm_skinny": [I, P, L, P, L, P, P, I, I, I, I, I, L, P],
+        "pae_gemm_skinny_rope": [P, L, P, L, P, P, I, I, I, I, I, I, I, P, P, P, P, I, I, P, P, P],
         "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "pae_sample": [P, P, L, P, P, I, I, P, P, P, P],
@@ -244,6 +245,40 @@ def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optio
     bp, bf = _param(bias)
     _check(library().pae_gemm_skinny(epilogue, out.data_ptr(), out.stride(-2), a.data_ptr(), a.stride(0),
                                      w.data_ptr(), bp, bf, M, N, K_, splits, M * N, _stream()))
+
+
+def skinny_rope_supported(a: torch.Tensor, w: torch.Tensor, hd: int, rot: int) -> bool:
+    """Whether `gemm_skinny_rope` takes this product: a skinny product whose head size and
+    rotated width are multiples of 16."""
+    return skinny_supported(a, w) and hd % 16 == 0 and rot % 16 == 0 and 0 <= rot <= hd
+
+
+def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], nh: int,
+                     nkv: int, hd: int, rot: int, inv_freq: Optional[torch.Tensor], positions: torch.Tensor,
+                     tok_seq: Optional[torch.Tensor], block_tables: Optional[torch.Tensor], block_size: int,
+                     k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor]) -> None:
+    """Query/key/value projection of at most 64 rows with the rotation and the cache write in its
+    epilogue: q_out[M, nh * hd] = rotated queries; rotated keys and raw values go to their slots
+    (nkv == 0: `w` holds the query rows only and nothing is stored)."""
+    _gpu(q_out, a, w, bias, inv_freq, positions, tok_seq, block_tables, k_cache, v_cache)
+    M, K_ = a.shape
+    assert skinny_rope_supported(a, w, hd, rot) and w.shape == ((nh + 2 * nkv) * hd, K_) and w.is_contiguous()
+    assert q_out.shape == (M, nh * hd) and q_out.dtype == torch.bfloat16 and q_out.stride(1) == 1
+    assert positions.dtype == torch.int32 and positions.numel() == M
+    if rot:
+        assert inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() == rot // 2
+    max_blocks = 0
+    if nkv:
+        assert k_cache.dtype == torch.bfloat16 == v_cache.dtype
+        assert tok_seq.dtype == torch.int32 and tok_seq.numel() == M
+        assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+        _check_pools(k_cache, v_cache, nkv, block_size, hd)
+        max_blocks = block_tables.shape[1]
+    bp, bf = _param(bias)
+    _check(library().pae_gemm_skinny_rope(q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(),
+                                          bp, bf, M, K_, nh, nkv, hd, rot, _ptr(inv_freq) if rot else None,
+                                          positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks,
+                                          block_size, _ptr(k_cache), _ptr(v_cache), _stream()))
 
 
 def gemm_plain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:

@@ -73,14 +73,20 @@ class PagedAttention(Part):
         group = ctx.cache.group_of(ctx.cache_entry)
         k_cache, v_cache = ctx.cache.kv_of(ctx.cache_entry)
         table = ctx.block_tables[group]
+        # a position encoding may offer the projection, its encoding and the cache write as one step
+        fused = getattr(self.position, "project_encode_store", None)
         if ctx.writes_cache:
-            qkv = self.qkv(x)
-            self.position.encode_and_store(ctx, qkv, s.num_heads, s.num_kv_heads, s.head_dim, k_cache, v_cache,
-                                           table, ctx.cache.block_size)
+            stored = (s.num_kv_heads, s.head_dim, k_cache, v_cache, table, ctx.cache.block_size)
+            qkv = fused(ctx, x, self.qkv, s.num_heads, *stored) if fused else None
+            if qkv is None:
+                qkv = self.qkv(x)
+                self.position.encode_and_store(ctx, qkv, s.num_heads, *stored)
         else:
-            qkv = self.q_only(x)
-            self.position.encode_and_store(ctx, qkv, s.num_heads, 0, s.head_dim, None, None, None,
-                                           ctx.cache.block_size)
+            stored = (0, s.head_dim, None, None, None, ctx.cache.block_size)
+            qkv = fused(ctx, x, self.q_only, s.num_heads, *stored) if fused else None
+            if qkv is None:
+                qkv = self.q_only(x)
+                self.position.encode_and_store(ctx, qkv, s.num_heads, *stored)
         attn = torch.empty((x.shape[0], s.num_heads * s.head_dim), dtype=x.dtype, device=x.device)
         geometry = (s.num_heads, s.num_kv_heads, s.head_dim, s.scale, s.window or 0)
         if K.mfma_attention_supported(x.dtype, s.num_heads, s.num_kv_heads, s.head_dim, ctx.cache.block_size) \

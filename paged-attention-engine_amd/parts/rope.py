@@ -34,6 +34,22 @@ class NeoxRope(Part):
                         block_table, block_size, k_cache, v_cache)
 
 
+    def project_encode_store(self, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
+        """The projection, the rotation and the cache write as one kernel, where there is one for
+        these sizes; otherwise None, and the caller runs the two steps."""
+        return _fused_projection(self.spec.rotary_dim, self.inv_freq, ctx, x, linear, nh, nkv, hd, k_cache,
+                                 v_cache, block_table, block_size)
+
+
+def _fused_projection(rot, inv_freq, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
+    if x.dtype != torch.bfloat16 or not K.skinny_rope_supported(x, linear.weight, hd, rot):
+        return None
+    q = torch.empty((x.shape[0], nh * hd), dtype=x.dtype, device=x.device)
+    K.gemm_skinny_rope(q, x, linear.weight, linear.bias, nh, nkv, hd, rot, inv_freq, ctx.positions, ctx.tok_seq,
+                       block_table, block_size, k_cache, v_cache)
+    return q
+
+
 @register_position_encoding("none")
 class NoPosition(Part):
     graph_safe = True
@@ -43,3 +59,6 @@ class NoPosition(Part):
         if k_cache is not None:
             K.rope_kv_write(qkv, nh, nkv, hd, 0, None, ctx.positions, ctx.tok_seq, block_table, block_size,
                             k_cache, v_cache)
+
+    def project_encode_store(self, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
+        return _fused_projection(0, None, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size)

@@ -247,6 +247,62 @@ def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs):
     assert torch.equal(d_kp.cpu()[untouched], kp[untouched])
 
 
+@pytest.mark.parametrize("M", [1, 7, 16, 23, 64])
+@pytest.mark.parametrize("nh,nkv,hd,rot,bs,Kdim,bias", [
+    (4, 2, 16, 16, 4, 72, True), (6, 1, 48, 48, 16, 136, False), (3, 3, 32, 16, 8, 264, True),
+    (5, 1, 64, 0, 16, 200, True), (12, 2, 128, 128, 16, 1536, True)])
+def test_gemm_skinny_rope(M, nh, nkv, hd, rot, bs, Kdim, bias):
+    """The projection with rotation and cache write in its epilogue against: a float64 product,
+    rounded to bfloat16 (as the separate projection would), rotated, and laid into the pools."""
+    torch.manual_seed(M + nh)
+    theta = 50000.0
+    # three sequences take turns; positions grow by 3 per row so that rows land in different pages
+    tok_seq = [t % 3 for t in range(M)]
+    positions = [2 + 3 * (t // 3) + 11 * (t % 3) for t in range(M)]
+    lens = [max([p for p, s in zip(positions, tok_seq) if s == q] + [0]) + 1 for q in range(3)]
+    num_blocks = sum(-(-n // bs) for n in lens) + 3
+    tables = scattered_tables(lens, bs, num_blocks, seed=5)
+    N = (nh + 2 * nkv) * hd
+    a = (torch.randn(M, Kdim) * 0.5).to(torch.bfloat16)
+    w = (torch.randn(N, Kdim) * 0.1).to(torch.bfloat16)
+    b = torch.randn(N).to(torch.bfloat16) if bias else None
+    kp = torch.full((num_blocks, nkv, bs, hd), 7.0, dtype=torch.bfloat16)
+    vp = torch.full((num_blocks, nkv, hd, bs), 7.0, dtype=torch.bfloat16)
+    d_kp, d_vp = kp.to(DEV), vp.to(DEV)
+    q = torch.full((M, nh * hd), 9.0, dtype=torch.bfloat16, device=DEV)
+    inv = plain.rope_inv_freq(rot, theta).to(DEV) if rot else None
+    K().gemm_skinny_rope(q, a.to(DEV), w.to(DEV), None if b is None else b.to(DEV), nh, nkv, hd, rot, inv,
+                         torch.tensor(positions, dtype=torch.int32, device=DEV),
+                         torch.tensor(tok_seq, dtype=torch.int32, device=DEV), tables.to(DEV), bs, d_kp, d_vp)
+    exact = a.double() @ w.double().t() + (0 if b is None else b.double())
+    x = exact.to(torch.bfloat16).double().view(M, nh + 2 * nkv, hd)
+    rotated = x.clone()
+    if rot:
+        cos, sin = plain.rope_cos_sin(plain.rope_inv_freq(rot, theta, torch.float64), torch.tensor(positions),
+                                      torch.float64)
+        rotated[..., :rot] = x[..., :rot] * cos[:, None] + plain.rotate_half(x[..., :rot]) * sin[:, None]
+    # one bfloat16 rounding of the product (values up to ~4 here) and one of the rotated value
+    bound = 2.0 ** -8 * max(1.0, float(exact.abs().max())) * 2.5
+    assert (q.cpu().double().view(M, nh, hd) - rotated[:, :nh]).abs().max() <= bound
+    want_k, want_v = kp.clone().double(), vp.clone().double()
+    touched = torch.zeros(num_blocks, dtype=torch.bool)
+    for t, (p, s) in enumerate(zip(positions, tok_seq)):
+        blk = int(tables[s, p // bs])
+        touched[blk] = True
+        want_k[blk, :, p % bs, :] = rotated[t, nh:nh + nkv]
+        want_v[blk, :, :, p % bs] = x[t, nh + nkv:]
+    assert (d_kp.cpu().double() - want_k).abs().max() <= bound
+    assert (d_vp.cpu().double() - want_v).abs().max() <= bound
+    # other pages keep what they held (other slots of touched pages are held to 7.0 by the bounds above)
+    assert torch.equal(d_kp.cpu()[~touched], kp[~touched]) and torch.equal(d_vp.cpu()[~touched], vp[~touched])
+    # queries only (a layer that reads another layer's cache): nothing is stored
+    q2 = torch.empty_like(q)
+    K().gemm_skinny_rope(q2, a.to(DEV), w[:nh * hd].contiguous().to(DEV), None if b is None else b[:nh * hd].to(DEV),
+                         nh, 0, hd, rot, inv, torch.tensor(positions, dtype=torch.int32, device=DEV), None, None, bs,
+                         None, None)
+    assert torch.equal(q2, q)
+
+
 # ------------------------------------------------------------------ attention
 def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=None, seed=0):
     """Queries are the last q_lens[s] positions of each sequence.  Returns (got, want)."""
