@@ -42,10 +42,6 @@ int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t 
                           const void* v_cache, const int* tiles, int num_tiles, const int* positions,
                           const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,
                           int window, hipStream_t stream);
-int pae_attn_prefill_long_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
-                               const void* v_cache, const int* tiles, int num_tiles, const int* positions,
-                               const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd,
-                               float scale, int window, hipStream_t stream);
 int pae_sample_chunks(int vocab);
 int pae_sample(int* tokens, const float* logits, int64_t ld, const float* temperature, const float* uniform,
                int num_rows, int vocab, float* chunk_max, int* chunk_arg, double* chunk_sum, hipStream_t stream);

@@ -16,7 +16,8 @@
 //          page is read once for all of them.  Four wavefronts take pages in turn
 //          and merge in LDS; the last workgroup to finish merges the splits.  Splits
 //          start at multiples of the split length from position 0.
-// prefill: one wavefront per (32 consecutive tokens of a sequence, query head).
+// prefill: one workgroup per (up to 64 consecutive tokens of a sequence, query head), whose
+//          wavefronts share out the keys (see there).
 //
 // Masking is the reference's rule (engine/attention.py:474-487: key j visible iff
 // j <= position of the query) plus an optional window.  A column's result depends
@@ -276,75 +277,274 @@ __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_s
 }
 
 // ------------------------------------------------------------------ prefill
-// tiles[t] = (row of the sequence in the tables, first flat token, number of tokens <= 32);
-// the tokens of a tile are consecutive in the step and in position.
-#define PREFILL_CT 2
-template <int HD>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+// One workgroup per (run of up to 16 CT consecutive tokens of a sequence, query head).  All four
+// wavefronts hold the run's queries (B operands of the first product) and take the keys in
+// turn, 32 at a time: wavefront w takes keys [lo + 32 (w + 4 i), + 32).  Every wavefront reads
+// its own keys and values straight from the cache into registers, so the loop has no barrier.
+// Keys and values have one register set each, refilled as soon as the product that read it has
+// been issued: the next keys arrive during the softmax and the second product, the next values
+// during the following first product.  At the end the four partial results (reference, sum,
+// unnormalised output) are merged through LDS, column tile ct by wavefront ct.
+//
+// The softmax keeps, per column, a reference value that is at most RESCALE_STEP (in units of log2)
+// below the largest score seen: weights are exp2(score - reference), at most 2^RESCALE_STEP, and the
+// sums so far are rescaled only when a score passes reference + RESCALE_STEP (then the reference
+// becomes the column's maximum).  Any reference gives the same quotient sum(w v) / sum(w); a stale
+// one saves rescaling the whole output tile for every 32 keys, which costs more than the products.
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+#define RESCALE_STEP 8.0f
+
+// A register loaded in the order (row = lane / 4, group = lane % 4), in which a quad of lanes reads
+// contiguous bytes, moved to the matrix instruction's order (row = lane % 16, group = lane / 16).
+__device__ __forceinline__ bf16x8 quad_to_mfma_order(bf16x8 x, int fetch_from) {
+  i32x4 raw = *reinterpret_cast<i32x4*>(&x);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) raw[i] = __builtin_amdgcn_ds_bpermute(fetch_from, raw[i]);
+  return *reinterpret_cast<bf16x8*>(&raw);
+}
+
+// tiles[t] = (table row of the sequence, first flat token, number of tokens <= 64); blockIdx.z picks
+// the part of 16 CT tokens of the run that this workgroup takes.
+// BS: the page size if it is 16 (the value rows' offsets are then constants), or 0 for any other.
+template <int HD, int CT, int BS>
+__global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ tiles,
-    int num_tiles, const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks,
-    int bs, int nh, int nkv, float scale_log2, int window) {
+    const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int bs, int nh,
+    int nkv, float scale_log2, int window) {
+  constexpr int UNIT = 32, TOK = 16 * CT;
+  if (BS) bs = BS;
+  __shared__ float s_acc[3][HD / 16][4][PAE_WAVE];
+  __shared__ float s_ml[3][2][PAE_WAVE];
+
   const int wave = threadIdx.x / PAE_WAVE, lane = threadIdx.x % PAE_WAVE;
-  const int tile_id = blockIdx.x * 4 + wave;
-  if (tile_id >= num_tiles) return;
-  const int head = blockIdx.y;
-  const int kvh = head / (nh / nkv);
-  const int seq_row = tiles[tile_id * 3], tok0 = tiles[tile_id * 3 + 1], ntok = tiles[tile_id * 3 + 2];
-  const int* table = block_tables + (int64_t)seq_row * max_blocks;
   const int col = lane % 16, g4 = lane / 16;
+  const int head = blockIdx.x, kvh = head / (nh / nkv);
+  const int seq_row = tiles[blockIdx.y * 3];
+  const int tok0 = tiles[blockIdx.y * 3 + 1] + blockIdx.z * TOK;
+  const int ntok = min(TOK, tiles[blockIdx.y * 3 + 2] - (int)blockIdx.z * TOK);
+  if (ntok <= 0) return;  // the whole workgroup
+  const int* table = block_tables + (int64_t)seq_row * max_blocks;
   const int pos0 = positions[tok0];
 
-  int pos[PREFILL_CT], start[PREFILL_CT];
-  bf16x8 qf[PREFILL_CT][HD / 32];
-  int lo = pos0, hi = pos0;  // keys any column needs: [lo, hi]
+  int pos[CT], start[CT];
 #pragma unroll
-  for (int ct = 0; ct < PREFILL_CT; ++ct) {
+  for (int ct = 0; ct < CT; ++ct) {
     const int c = ct * 16 + col;
     const bool live = c < ntok;
     pos[ct] = live ? pos0 + c : -1;  // a dead column sees no key
     start[ct] = (live && window > 0 && pos[ct] - window + 1 > 0) ? pos[ct] - window + 1 : 0;
-    const bf16_t* qrow = q + (int64_t)(tok0 + (live ? c : 0)) * q_stride + (int64_t)head * HD;
+  }
+  bf16x8 qf[CT][HD / 32];  // B operands of the first product: column tile ct, features 32 j ..
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int c = ct * 16 + col;
+    const bf16_t* qrow = q + (int64_t)(tok0 + (c < ntok ? c : 0)) * q_stride + (int64_t)head * HD;
 #pragma unroll
     for (int j = 0; j < HD / 32; ++j) qf[ct][j] = *reinterpret_cast<const bf16x8*>(qrow + 32 * j + 8 * g4);
   }
-  hi = pos0 + ntok - 1;
-  lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int hi = pos0 + ntok - 1;                                                        // last key any token sees
+  const int lo = (window > 0 && pos0 - window + 1 > 0) ? (pos0 - window + 1) / UNIT * UNIT : 0;  // first, rounded down
+  const int last_start = (window > 0 && hi - window + 1 > 0) ? hi - window + 1 : 0;     // window start of the last token
 
-  AttnState<HD, PREFILL_CT> st;
+  f32x4 acc[CT][HD / 16];  // O^T: rows hd = 16 t + 4 g4 + i, column = lane % 16
+  float ref[CT], l[CT];    // the column's reference (log2 units) and this lane's share of its sum of weights
 #pragma unroll
-  for (int ct = 0; ct < PREFILL_CT; ++ct) {
-    st.m[ct] = NEG_BIG;
-    st.l[ct] = 0.f;
+  for (int ct = 0; ct < CT; ++ct) {
+    ref[ct] = NEG_BIG;
+    l[ct] = 0.f;
 #pragma unroll
-    for (int t = 0; t < HD / 16; ++t) st.acc[ct][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < HD / 16; ++t) acc[ct][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
+
+  // Loads in the order (row = lane / 4, group = lane % 4): a quad reads 64 contiguous bytes of a
+  // key row, or 32 of a value row.  kf[p][j]: keys of page p, features 32 j ..; vf[t]: features
+  // 16 t .., whose 8 k slots per lane are keys 4 g4 .. + 3 of the first page followed by the same
+  // four of the second, exactly the scores a lane holds after the first product.
+  const int lrow = lane / 4, lgrp = lane % 4;
+  const int fetch_from = ((lane % 16) * 4 + lane / 16) * 4;
   const int page_elems = bs * HD;
-  bf16x8 kf[HD / 32];
-  s16x4 vf[HD / 16];
-  for (int key0 = lo / 16 * 16; key0 <= hi; key0 += 16) {
-    const int blk = table[key0 / bs];
-    const int64_t base = ((int64_t)blk * nkv + kvh) * page_elems;
-    load_kv_tile<HD>(kf, vf, k_cache + base + (int64_t)(key0 % bs) * HD, v_cache + base + key0 % bs, bs);
-    kv_to_mfma_order<HD>(kf, vf);
-    attn_tile<HD, PREFILL_CT>(st, kf, vf, qf, key0, pos, start, scale_log2);
-  }
+  bf16x8 kf[2][HD / 32], vf[HD / 16];
+  auto page_base = [&](int key0, int p) -> int64_t {
+    const int key = key0 + 16 * p;
+    const int kc = key <= hi ? key : key0;  // a tile past the end repeats the first one (all of it is masked)
+    // a page the window has passed was given back (its entry is -1): all its keys are masked, read page 0
+    return ((int64_t)max(table[kc / bs], 0) * nkv + kvh) * page_elems;
+  };
+  auto load_keys = [&](int key0) {
 #pragma unroll
-  for (int ct = 0; ct < PREFILL_CT; ++ct) {
-    float l = st.l[ct];
-    l += __shfl_xor(l, 16, PAE_WAVE);
-    l += __shfl_xor(l, 32, PAE_WAVE);
-    const int c = ct * 16 + col;
-    if (c >= ntok) continue;
-    const float inv = 1.0f / l;
-    bf16_t* o = out + (int64_t)(tok0 + c) * out_stride + (int64_t)head * HD;
+    for (int p = 0; p < 2; ++p) {
+      const int key = key0 + 16 * p, kc = key <= hi ? key : key0;
+      const bf16_t* kp = k_cache + page_base(key0, p) + (int64_t)(kc % bs) * HD;
+#pragma unroll
+      for (int j = 0; j < HD / 32; ++j) kf[p][j] = *reinterpret_cast<const bf16x8*>(kp + lrow * HD + 32 * j + 8 * lgrp);
+    }
+  };
+  auto load_values = [&](int key0) {
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      const int key = key0 + 16 * p, kc = key <= hi ? key : key0;
+      const bf16_t* vp = v_cache + page_base(key0, p) + kc % bs;
+#pragma unroll
+      for (int t = 0; t < HD / 16; ++t)
+        reinterpret_cast<bf16x4*>(&vf[t])[p] = *reinterpret_cast<const bf16x4*>(vp + (int64_t)(16 * t + lrow) * bs + 4 * lgrp);
+    }
+  };
+
+  int key0 = lo + UNIT * wave;  // the same in every lane of a wavefront: the branches on it are uniform
+  if (key0 <= hi) {
+    load_keys(key0);
+    load_values(key0);
+  }
+  for (; key0 <= hi; key0 += 4 * UNIT) {
+    const bool more = key0 + 4 * UNIT <= hi;
+    // The queries stay in the accumulation registers, which the matrix instruction reads directly:
+    // the other half of the register file is needed for the keys, values and scores in flight.
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int j = 0; j < HD / 32; ++j) asm volatile("" : "+a"(qf[ct][j]));
+    // scores of the 32 keys for every column tile
+    f32x4 s[CT][2];
+    {
+      bf16x8 ka[2][HD / 32];
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int j = 0; j < HD / 32; ++j) ka[p][j] = quad_to_mfma_order(kf[p][j], fetch_from);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          s[ct][p] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int j = 0; j < HD / 32; ++j)
+            s[ct][p] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[p][j], qf[ct][j], s[ct][p], 0, 0, 0);
+        }
+    }
+    if (more) load_keys(key0 + 4 * UNIT);  // into the registers the first product has just read
+    if (!(key0 + UNIT - 1 <= pos0 && key0 >= last_start)) {  // some key is hidden from some token of the run
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = key0 + 16 * p + 4 * g4 + i;
+            if (!(key <= pos[ct] && key >= start[ct])) s[ct][p][i] = -INFINITY;
+          }
+    }
+    // does any score pass its column's reference by more than the step?  (each lane for its own scores)
+    float mx[CT];
+    bool passed = false;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      mx[ct] = fmaxf(fmaxf(fmaxf(s[ct][0][0], s[ct][0][1]), fmaxf(s[ct][0][2], s[ct][0][3])),
+                     fmaxf(fmaxf(s[ct][1][0], s[ct][1][1]), fmaxf(s[ct][1][2], s[ct][1][3]))) * scale_log2;
+      passed |= mx[ct] > ref[ct] + RESCALE_STEP;
+    }
+    if (__builtin_amdgcn_ballot_w64(passed) != 0) {  // the same in every lane; rare after the first units
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int t = 0; t < HD / 16; ++t) asm volatile("" : "+a"(acc[ct][t]));  // moved from there only in here
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        float m = fmaxf(mx[ct], NEG_BIG);
+        m = fmaxf(m, __shfl_xor(m, 16, PAE_WAVE));
+        m = fmaxf(m, __shfl_xor(m, 32, PAE_WAVE));  // the column's maximum in this unit
+        const float to = m > ref[ct] + RESCALE_STEP ? m : ref[ct];
+        const float alpha = __builtin_amdgcn_exp2f(ref[ct] - to);
+        ref[ct] = to;
+        l[ct] *= alpha;
+#pragma unroll
+        for (int t = 0; t < HD / 16; ++t) acc[ct][t] *= alpha;
+      }
+    }
+    // the sums are in the accumulation registers on both ways here (or the compiler moves the whole
+    // output tile to ordinary registers and back in every pass for the sake of the rare branch)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int t = 0; t < HD / 16; ++t) asm volatile("" : "+a"(acc[ct][t]));
+    bf16x8 pb[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      float w[8];
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          w[4 * p + i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ct][p][i], scale_log2, -ref[ct]));
+      l[ct] += ((w[0] + w[1]) + (w[2] + w[3])) + ((w[4] + w[5]) + (w[6] + w[7]));
+      bf16x2* pairs = reinterpret_cast<bf16x2*>(&pb[ct]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pairs[i] = __builtin_convertvector((f32x2){w[2 * i], w[2 * i + 1]}, bf16x2);
+    }
 #pragma unroll
     for (int t = 0; t < HD / 16; ++t) {
-      s16x4 w;
+      const bf16x8 va = quad_to_mfma_order(vf[t], fetch_from);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) w[i] = bf16_bits(st.acc[ct][t][i] * inv);
-      *reinterpret_cast<s16x4*>(o + 16 * t + 4 * g4) = w;
+      for (int ct = 0; ct < CT; ++ct) acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[ct], acc[ct][t], 0, 0, 0);
     }
+    if (more) load_values(key0 + 4 * UNIT);
+  }
+
+  // merge: column tile ct is summed by wavefront ct from its own state and the three others' in LDS
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    float sum = l[ct];
+    sum += __shfl_xor(sum, 16, PAE_WAVE);
+    sum += __shfl_xor(sum, 32, PAE_WAVE);
+    l[ct] = sum;
+  }
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int merger = ct % 4;
+    if (wave != merger) {
+      const int slot = wave < merger ? wave : wave - 1;
+#pragma unroll
+      for (int t = 0; t < HD / 16; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_acc[slot][t][i][lane] = acc[ct][t][i];
+      s_ml[slot][0][lane] = ref[ct];
+      s_ml[slot][1][lane] = l[ct];
+    }
+    __syncthreads();
+    if (wave == merger) {
+      float m = ref[ct];
+#pragma unroll
+      for (int w = 0; w < 3; ++w) m = fmaxf(m, s_ml[w][0][lane]);
+      const float own = exp2f(ref[ct] - m);
+      float sum = l[ct] * own;
+      float scale_w[3];
+#pragma unroll
+      for (int w = 0; w < 3; ++w) {
+        scale_w[w] = exp2f(s_ml[w][0][lane] - m);
+        sum += s_ml[w][1][lane] * scale_w[w];
+      }
+      const int c = ct * 16 + col;
+      if (c < ntok) {
+        const float inv = 1.0f / sum;
+        bf16_t* o = out + (int64_t)(tok0 + c) * out_stride + (int64_t)head * HD;
+#pragma unroll
+        for (int t = 0; t < HD / 16; ++t) {
+          s16x4 w4;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float a = acc[ct][t][i] * own;
+#pragma unroll
+            for (int w = 0; w < 3; ++w) a += s_acc[w][t][i][lane] * scale_w[w];
+            w4[i] = bf16_bits(a * inv);
+          }
+          *reinterpret_cast<s16x4*>(o + 16 * t + 4 * g4) = w4;
+        }
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -402,229 +602,31 @@ extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q
   return pae_check_launch("attn_decode");
 }
 
+// tiles[t] = (table row of the sequence, first flat token, number of tokens <= 64), heaviest runs
+// first: workgroups start in the order of the grid, and the last to finish sets the time.
 extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
-                                     const void* k_cache, const void* v_cache, const int* tiles, int num_tiles,
-                                     const int* positions, const int* block_tables, int max_blocks, int bs,
-                                     int nh, int nkv, int hd, float scale, int window, hipStream_t stream) {
-  if (int rc = check_common("attn_prefill", nh, nkv, hd, bs, max_blocks, window)) return rc;
-  PAE_REQUIRE(nh <= 65535, "attn_prefill: grid too large");
-  if (num_tiles <= 0) return 0;
-  const float scale_log2 = scale * LOG2E;
-  dim3 grid((num_tiles + 3) / 4, nh);
-#define CALL(HD)                                                                                          \
-  attn_prefill_kernel<HD><<<grid, 256, 0, stream>>>((bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, \
-                                                    (const bf16_t*)k_cache, (const bf16_t*)v_cache, tiles, \
-                                                    num_tiles, positions, block_tables, max_blocks, bs, nh, \
-                                                    nkv, scale_log2, window)
-  FOR_HEAD_DIM(hd, CALL)
-#undef CALL
-  return pae_check_launch("attn_prefill");
-}
-
-// ------------------------------------------------------------------ prefill, long runs
-// One workgroup per (up to 128 consecutive tokens of a sequence, query head); each of
-// its four wavefronts owns 32 of the tokens.  Keys and values of BN keys at a time are
-// staged in LDS by the whole workgroup (the next tile is fetched into registers while
-// the current one is used) and every wavefront multiplies them with its own queries:
-//   S^T[32 keys x 32 tokens] = K * Q^T             (MFMA 32x32x16, k = hd)
-//   O^T[32 features x 32 tokens] += V^T * P^T      (MFMA 32x32x16, k = 16 keys)
-// The accumulator of S^T holds, per lane (token = lane % 32, half = lane / 32), keys
-// 8 j + 4 half + i of each 32-key block; two such groups of four are the 8 k-slots of a
-// lane in the second product, whose A operand reads the values of exactly those keys.
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-
-template <int HD, int BN>
-__global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_lds_kernel(
-    bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
-    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ tiles,
-    const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int bs, int nh,
-    int nkv, float scale_log2, int window) {
-  constexpr int KS = HD + 8;   // row stride of the key tile in LDS (elements), padded against bank conflicts
-  constexpr int VS = BN + 8;   // row stride of the transposed value tile
-  constexpr int PAGES = BN / 16;
-  constexpr int KCH = (16 * HD / 8 + 255) / 256;  // 16-byte chunks per thread and page
-  __shared__ __attribute__((aligned(16))) bf16_t k_lds[BN * KS];
-  __shared__ __attribute__((aligned(16))) bf16_t v_lds[HD * VS];
-
-  const int tid = threadIdx.x, wave = tid / PAE_WAVE, lane = tid % PAE_WAVE;
-  const int col = lane % 32, half = lane / 32;
-  const int head = blockIdx.y, kvh = head / (nh / nkv);
-  const int seq_row = tiles[blockIdx.x * 3], tok0 = tiles[blockIdx.x * 3 + 1], ntok = tiles[blockIdx.x * 3 + 2];
-  const int* table = block_tables + (int64_t)seq_row * max_blocks;
-  const int pos0 = positions[tok0];
-  const int c = wave * 32 + col;          // this lane's token within the tile
-  const bool live = c < ntok;
-  const int pos = live ? pos0 + c : -1;   // a dead column sees no key
-  const int start = (live && window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int wave_hi = min(pos0 + wave * 32 + 31, pos0 + ntok - 1);  // last position of this wavefront
-  const bool wave_live = wave * 32 < ntok;
-  const bool wave_full = wave * 32 + 32 <= ntok;  // no dead column in this wavefront
-  const int wave_lo = pos0 + wave * 32;            // its first position, and the window start of its last
-  const int wave_start = (window > 0 && wave_hi - window + 1 > 0) ? wave_hi - window + 1 : 0;
-  const int lo = (window > 0 && pos0 - window + 1 > 0) ? (pos0 - window + 1) / BN * BN : 0;
-  const int hi = pos0 + ntok - 1;
-
-  // queries: B operand, lane holds token `col`, features 16 ks + 8 half .. + 7
-  bf16x8 qf[HD / 16];
-  {
-    const bf16_t* qrow = q + (int64_t)(tok0 + (live ? c : 0)) * q_stride + (int64_t)head * HD;
-#pragma unroll
-    for (int ks = 0; ks < HD / 16; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + 16 * ks + 8 * half);
-  }
-  f32x16 acc[HD / 32];
-#pragma unroll
-  for (int t = 0; t < HD / 32; ++t)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
-  float m = NEG_BIG, l = 0.f;
-
-  const int page_elems = bs * HD;
-  // staging registers: per page, this thread's 16-byte chunks of the key page and of the value page
-  bf16x8 kreg[PAGES][KCH], vreg[PAGES][KCH];
-  auto fetch = [&](int key0) {
-#pragma unroll
-    for (int p = 0; p < PAGES; ++p) {
-      const int key = key0 + 16 * p;
-      const int kc = key <= hi ? key : key0;  // pages past the end repeat the first one (never used)
-      // a page the window has passed was given back (its entry is -1): every key of it is masked, read page 0
-      const int64_t base = ((int64_t)max(table[kc / bs], 0) * nkv + kvh) * page_elems;
-      const bf16_t* kp = k_cache + base + (int64_t)(kc % bs) * HD;  // [16 keys][HD], contiguous
-      const bf16_t* vp = v_cache + base + kc % bs;                  // [HD][bs]: 16 keys of each feature
-#pragma unroll
-      for (int ch = 0; ch < KCH; ++ch) {
-        const int idx = tid + 256 * ch;  // chunk index within the page: 16 * HD / 8 chunks
-        if (idx < 16 * HD / 8) {
-          kreg[p][ch] = *reinterpret_cast<const bf16x8*>(kp + idx * 8);
-          const int d = idx / 2, part = idx % 2;  // feature, which 8 of the 16 keys
-          vreg[p][ch] = *reinterpret_cast<const bf16x8*>(vp + (int64_t)d * bs + 8 * part);
-        }
-      }
-    }
-  };
-  auto stage = [&]() {
-#pragma unroll
-    for (int p = 0; p < PAGES; ++p)
-#pragma unroll
-      for (int ch = 0; ch < KCH; ++ch) {
-        const int idx = tid + 256 * ch;
-        if (idx < 16 * HD / 8) {
-          const int key = idx / (HD / 8), kchunk = idx % (HD / 8);
-          *reinterpret_cast<bf16x8*>(k_lds + (16 * p + key) * KS + 8 * kchunk) = kreg[p][ch];
-          const int d = idx / 2, part = idx % 2;
-          *reinterpret_cast<bf16x8*>(v_lds + d * VS + 16 * p + 8 * part) = vreg[p][ch];
-        }
-      }
-  };
-
-  fetch(lo);
-  for (int key0 = lo; key0 <= hi; key0 += BN) {
-    __syncthreads();  // the previous tile has been read by every wavefront
-    stage();
-    __syncthreads();
-    if (key0 + BN <= hi) fetch(key0 + BN);
-    if (!wave_live || key0 > wave_hi) continue;  // nothing for this wavefront in the tile (causal)
-    // scores of the whole tile first, then one softmax update and one rescale for it
-    f32x16 s[BN / 32];
-#pragma unroll
-    for (int kb = 0; kb < BN / 32; ++kb) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
-      bf16x8 kf[HD / 16];  // all key fragments of the block are read before the first product uses one
-#pragma unroll
-      for (int ks = 0; ks < HD / 16; ++ks)
-        kf[ks] = *reinterpret_cast<const bf16x8*>(k_lds + (32 * kb + col) * KS + 16 * ks + 8 * half);
-#pragma unroll
-      for (int ks = 0; ks < HD / 16; ++ks) s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], s[kb], 0, 0, 0);
-    }
-    // a tile that every token of this wavefront sees whole needs no mask
-    const bool whole = wave_full && key0 + BN - 1 <= wave_lo && key0 >= wave_start;
-    float mx = NEG_BIG;
-    if (whole) {
-#pragma unroll
-      for (int kb = 0; kb < BN / 32; ++kb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          s[kb][v] *= scale_log2;
-          mx = fmaxf(mx, s[kb][v]);
-        }
-    } else {
-#pragma unroll
-      for (int kb = 0; kb < BN / 32; ++kb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int key = key0 + 32 * kb + 8 * (v / 4) + 4 * half + v % 4;
-          s[kb][v] = (key <= pos && key >= start) ? s[kb][v] * scale_log2 : -INFINITY;
-          mx = fmaxf(mx, s[kb][v]);
-        }
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, PAE_WAVE));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = exp2f(m - m_new);
-    m = m_new;
-    float psum = 0.f;
-    bf16x8 pb[BN / 32][2];
-#pragma unroll
-    for (int kb = 0; kb < BN / 32; ++kb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float p = exp2f(s[kb][v] - m_new);
-        psum += p;
-        pb[kb][v / 8][v % 8] = (__bf16)p;
-      }
-    l = l * alpha + psum;
-#pragma unroll
-    for (int t = 0; t < HD / 32; ++t) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[t][v] *= alpha;
-      // value fragments: keys 16 st + 4 half + (0..3) and 16 st + 8 + 4 half + (0..3) of block kb, feature 32 t + col
-      bf16x8 vf[BN / 32][2];
-#pragma unroll
-      for (int kb = 0; kb < BN / 32; ++kb)
-#pragma unroll
-        for (int st = 0; st < 2; ++st) {
-          const bf16_t* vrow = v_lds + (32 * t + col) * VS + 32 * kb + 16 * st + 4 * half;
-          s16x4* dst = reinterpret_cast<s16x4*>(&vf[kb][st]);
-          dst[0] = *reinterpret_cast<const s16x4*>(vrow);
-          dst[1] = *reinterpret_cast<const s16x4*>(vrow + 8);
-        }
-#pragma unroll
-      for (int kb = 0; kb < BN / 32; ++kb)
-#pragma unroll
-        for (int st = 0; st < 2; ++st)
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[kb][st], pb[kb][st], acc[t], 0, 0, 0);
-    }
-  }
-  l += __shfl_xor(l, 32, PAE_WAVE);
-  if (!live) return;
-  const float inv = 1.0f / l;
-  bf16_t* o = out + (int64_t)(tok0 + c) * out_stride + (int64_t)head * HD;
-#pragma unroll
-  for (int t = 0; t < HD / 32; ++t)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {  // registers 4 j .. 4 j + 3 are features 32 t + 8 j + 4 half + (0..3)
-      s16x4 w;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) w[i] = bf16_bits(acc[t][4 * j + i] * inv);
-      *reinterpret_cast<s16x4*>(o + 32 * t + 8 * j + 4 * half) = w;
-    }
-}
-
-// tiles[t] = (table row of the sequence, first flat token, number of tokens <= 128)
-extern "C" int pae_attn_prefill_long_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                           const void* k_cache, const void* v_cache, const int* tiles,
                                           int num_tiles, const int* positions, const int* block_tables,
                                           int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
                                           hipStream_t stream) {
-  if (int rc = check_common("attn_prefill_long", nh, nkv, hd, bs, max_blocks, window)) return rc;
-  PAE_REQUIRE(nh <= 65535, "attn_prefill_long: grid too large");
+  if (int rc = check_common("attn_prefill", nh, nkv, hd, bs, max_blocks, window)) return rc;
+  PAE_REQUIRE(num_tiles <= 65535, "attn_prefill: %d runs exceed the grid", num_tiles);
   if (num_tiles <= 0) return 0;
   const float scale_log2 = scale * LOG2E;
-  dim3 grid(num_tiles, nh);
-#define CALL(HD)                                                                                            \
-  attn_prefill_lds_kernel<HD, (HD <= 128 ? 64 : 32)><<<grid, 256, 0, stream>>>(                             \
-      (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, \
+  // four column tiles (64 tokens) per workgroup up to head_dim 128, two above (registers)
+#define SPLIT_CT 4
+#define LAUNCH(HD, BS)                                                                                         \
+  attn_prefill_split_kernel<HD, SPLIT_CT, BS><<<dim3(nh, num_tiles, 4 / SPLIT_CT), 256, 0, stream>>>( \
+      (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,    \
       tiles, positions, block_tables, max_blocks, bs, nh, nkv, scale_log2, window)
+#define CALL(HD)        \
+  if (bs == 16) {       \
+    LAUNCH(HD, 16);     \
+  } else {              \
+    LAUNCH(HD, 0);      \
+  }
   FOR_HEAD_DIM(hd, CALL)
 #undef CALL
-  return pae_check_launch("attn_prefill_long");
+#undef LAUNCH
+  return pae_check_launch("attn_prefill");
 }

@@ -23,7 +23,7 @@ from ..parts import StepContext
 from .model import Model
 
 
-from ..kernels.lib import LONG_TILE, SHORT_TILE  # tokens per run of the two prefill attention kernels
+from ..kernels.lib import PREFILL_TILE  # tokens per run of the prefill attention kernel
 
 
 @dataclass(frozen=True)
@@ -105,14 +105,15 @@ class StepRunner:
         T, S = len(ids), len(seq_ids)
         decode_only = self.use_graphs and T == S and (self.model.dtype == torch.float32 or S <= 64)
         decode_tokens = [q_starts[i] for i in range(S) if q_lens[i] == 1]
-        tiles: List[int] = []
-        long_tiles: List[int] = []
+        runs = []  # (keys the run sees, tile): runs of at most PREFILL_TILE consecutive tokens of a sequence
         for i in range(S):
-            if q_lens[i] > SHORT_TILE:
-                for first in range(0, q_lens[i], LONG_TILE):
-                    long_tiles += [i, q_starts[i] + first, min(LONG_TILE, q_lens[i] - first)]
-            elif q_lens[i] > 1:
-                tiles += [i, q_starts[i], q_lens[i]]
+            if q_lens[i] > 1:
+                for first in range(0, q_lens[i], PREFILL_TILE):
+                    count = min(PREFILL_TILE, q_lens[i] - first)
+                    runs.append((past_lens[i] + first + count, [i, q_starts[i] + first, count]))
+        # the runs with the most keys start first: the last workgroup to finish sets the kernel's time
+        runs.sort(key=lambda run: -run[0])
+        tiles: List[int] = [x for _, tile in runs for x in tile]
         tables = []
         for group in cache.groups:
             per_seq = [cache.block_table(group.index, s) for s in seq_ids]
@@ -122,7 +123,7 @@ class StepRunner:
             tables.append((width, per_seq))
 
         # one staging buffer, one copy to the device
-        flat: List[int] = ids + positions + tok_seq + slots + rows + decode_tokens + tiles + long_tiles
+        flat: List[int] = ids + positions + tok_seq + slots + rows + decode_tokens + tiles
         for width, per_seq in tables:
             for table in per_seq:
                 flat.extend(table)
@@ -152,7 +153,6 @@ class StepRunner:
 
         d_ids, d_pos, d_seq, d_slots, d_rows = take(T), take(T), take(T), take(S), take(len(rows))
         d_decode, d_tiles = take(len(decode_tokens)), take(len(tiles)).view(-1, 3)
-        d_long = take(len(long_tiles)).view(-1, 3)
         block_tables: Dict[int, torch.Tensor] = {}
         for group, (width, _) in zip(cache.groups, tables):
             block_tables[group.index] = take(S * width).view(S, width)
@@ -161,7 +161,7 @@ class StepRunner:
                           positions=d_pos, tok_seq=d_seq, block_tables=block_tables, slots=d_slots,
                           cache=cache, seq_ids=seq_ids, q_starts=q_starts, q_lens=q_lens,
                           past_lens=past_lens, host_slots=slots, decode_tokens=d_decode,
-                          prefill_tiles=d_tiles, prefill_long_tiles=d_long)
+                          prefill_tiles=d_tiles)
         if captured is None:
             return self.model.forward(ctx, d_ids, d_rows)
         if captured.graph is None:

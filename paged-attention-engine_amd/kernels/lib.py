@@ -65,7 +65,6 @@ def _declare(lib) -> None:
         "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, P, P],
         "pae_attn_decode_split": [],
         "pae_attn_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
-        "pae_attn_prefill_long_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -344,16 +343,16 @@ def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cac
         part_acc.data_ptr(), part_ml.data_ptr(), _stream()))
 
 
-SHORT_TILE = 32    # tokens per run of the direct prefill kernel (one wavefront each)
-LONG_TILE = 128    # tokens per run of the LDS-staged prefill kernel (one workgroup each)
+PREFILL_TILE = 64  # tokens per run of the prefill attention kernel (one workgroup each)
 
 
 def attn_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                  tiles: torch.Tensor, positions: torch.Tensor, block_tables: torch.Tensor,
-                 nh: int, nkv: int, hd: int, scale: float, window: int, long: bool = False) -> None:
+                 nh: int, nkv: int, hd: int, scale: float, window: int) -> None:
     """Attention of runs of consecutive tokens; tiles[t] = (table row of the sequence, first
-    flat token, number of tokens): up to 32 tokens a run, or with `long` up to 128 (keys and
-    values are then staged in LDS for the whole workgroup)."""
+    flat token, number of tokens <= PREFILL_TILE).  One workgroup per run and head, whose
+    wavefronts share out the keys; workgroups start in the order of `tiles`, so the runs with
+    the most keys should come first."""
     _gpu(out, q, k_cache, v_cache, tiles, positions, block_tables)
     bs = k_cache.shape[2]
     assert q.dtype == torch.bfloat16 == out.dtype == k_cache.dtype and q.stride(1) == 1 and out.stride(1) == 1
@@ -362,8 +361,7 @@ def attn_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_ca
     assert tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.is_contiguous()
     assert positions.dtype == torch.int32 and positions.numel() == q.shape[0]
     assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
-    entry = library().pae_attn_prefill_long_bf16 if long else library().pae_attn_prefill_bf16
-    _check(entry(
+    _check(library().pae_attn_prefill_bf16(
         out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
         tiles.data_ptr(), tiles.shape[0], positions.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
         bs, nh, nkv, hd, float(scale), int(window), _stream()))

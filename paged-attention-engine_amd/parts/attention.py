@@ -96,9 +96,6 @@ class PagedAttention(Part):
                               *geometry)
             if ctx.prefill_tiles.numel():
                 K.attn_prefill(attn, qkv, k_cache, v_cache, ctx.prefill_tiles, ctx.positions, table, *geometry)
-            if ctx.prefill_long_tiles is not None and ctx.prefill_long_tiles.numel():
-                K.attn_prefill(attn, qkv, k_cache, v_cache, ctx.prefill_long_tiles, ctx.positions, table,
-                               *geometry, long=True)
         else:
             K.paged_attention_generic(attn, qkv, k_cache, v_cache, ctx.positions, ctx.tok_seq, table, *geometry)
         return self.out.branch(attn)

@@ -58,8 +58,7 @@ class StepContext:
     # consecutive tokens of sequences that bring 2..32, and runs of up to 128 of those that
     # bring more, each as (table row, first flat token, count)
     decode_tokens: Optional[torch.Tensor] = None   # int32 [number of single-token sequences]
-    prefill_tiles: Optional[torch.Tensor] = None   # int32 [number of short runs, 3]
-    prefill_long_tiles: Optional[torch.Tensor] = None  # int32 [number of long runs, 3]
+    prefill_tiles: Optional[torch.Tensor] = None   # int32 [runs of 2..64 tokens, 3]: table row, first token, count
     # set by the model for the stop that is running
     entry: int = 0                     # index in the schedule
     cache_entry: int = 0               # the stop whose cache is read (entry itself unless it borrows)

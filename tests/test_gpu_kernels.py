@@ -304,7 +304,7 @@ def test_gemm_skinny_rope(M, nh, nkv, hd, rot, bs, Kdim, bias):
 
 
 # ------------------------------------------------------------------ attention
-def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=None, seed=0):
+def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=None, seed=0, ramp=None):
     """Queries are the last q_lens[s] positions of each sequence.  Returns (got, want)."""
     torch.manual_seed(seed)
     num_blocks = sum(-(-n // bs) for n in seq_lens) + 5
@@ -323,6 +323,11 @@ def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=
         direction /= direction.norm()
         keys[0][key_pos] = 6.0 * direction * math.sqrt(hd) ** 0.5
         q[q_lens[0] - 1] = 6.0 * direction * math.sqrt(hd) ** 0.5
+    if ramp is not None:  # scores of sequence 0 climb by `ramp` (natural-log units) per key, up or down
+        direction = torch.randn(hd)
+        direction /= direction.norm()
+        keys[0] += (ramp * torch.arange(seq_lens[0]).float())[:, None, None] * direction * math.sqrt(hd) ** 0.5
+        q[:q_lens[0]] += direction * math.sqrt(hd) ** 0.5
     scale = hd ** -0.5
     q, keys, values = q.to(DT[dtype]), [k.to(DT[dtype]) for k in keys], [v.to(DT[dtype]) for v in values]
     want = torch.stack([reference_attention(q[t].float(), keys[s].float(), values[s].float(), p, scale, window)
@@ -337,17 +342,11 @@ def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=
     else:
         starts = [sum(q_lens[:s]) for s in range(len(q_lens))]
         dec = [starts[s] for s in range(len(q_lens)) if q_lens[s] == 1]
-        tiles, long_tiles = [], []
+        tiles = []
         for s, ql in enumerate(q_lens):
-            if ql > 32 and kind != "mfma_short":
-                for first in range(0, ql, 128):
-                    long_tiles.append([s, starts[s] + first, min(128, ql - first)])
-            elif ql > 1:
-                for first in range(0, ql, 32):
-                    tiles.append([s, starts[s] + first, min(32, ql - first)])
-        if long_tiles:
-            K().attn_prefill(out, qd, d(kp), d(vp), d(long_tiles, torch.int32), pos_d, tab_d, nh, nkv, hd, scale,
-                             window, long=True)
+            if ql > 1:
+                for first in range(0, ql, K().PREFILL_TILE):
+                    tiles.append([s, starts[s] + first, min(K().PREFILL_TILE, ql - first)])
         if dec:
             K().attn_decode(out, qd, d(kp), d(vp), d(dec, torch.int32), pos_d, seq_d, tab_d, nh, nkv, hd, scale, window)
         if tiles:
@@ -393,11 +392,20 @@ def test_one_far_key_stands_out(kind, key_pos, window, seen):
         assert want[0].abs().max() > 0.5
 
 
-@pytest.mark.parametrize("kind", ["mfma", "mfma_short"])
-@pytest.mark.parametrize("q_len", [2, 31, 32, 33, 64, 100, 128, 129, 300])
-def test_matrix_core_prefill_from_empty_and_warm(kind, q_len):
-    got, want = run_attention(kind, "bfloat16", 12, 2, 128, 16, 0, [q_len, 200 + q_len], [q_len, q_len])
+@pytest.mark.parametrize("q_len", [2, 31, 32, 33, 64, 65, 100, 128, 129, 300])
+def test_matrix_core_prefill_from_empty_and_warm(q_len):
+    got, want = run_attention("mfma", "bfloat16", 12, 2, 128, 16, 0, [q_len, 200 + q_len], [q_len, q_len])
     assert (got - want).abs().max() <= 3e-2
+
+
+@pytest.mark.parametrize("ramp", [0.02, 0.15, 0.5, -0.15])
+def test_matrix_core_prefill_rising_scores(ramp):
+    """The prefill kernel rescales its sums only when a score passes the running reference by 2^8:
+    scores that climb slowly (never rescaled, weights grow to the limit), quickly (rescaled in
+    nearly every 32 keys) or fall must all give the plain softmax."""
+    got, want = run_attention("mfma", "bfloat16", 6, 2, 128, 16, 0, [700, 50], [700, 50], ramp=ramp)
+    err = (got - want).abs().max(dim=1).values
+    assert float(err.max()) <= 3e-2, f"worst rows: {torch.topk(err, 5)}"
 
 
 @pytest.mark.parametrize("nh,nkv,hd,bs,window", MFMA_SHAPES)

@@ -37,8 +37,7 @@ def make_ctx(cache, dtype, seq_ids, q_lens):
         tables[group.index] = torch.tensor([list(r) + [-1] * (width - len(r)) for r in rows], dtype=torch.int32, device=DEV)
     slots = [cache.slot_of(s) for s in seq_ids]
     dec = [q_starts[i] for i, n in enumerate(q_lens) if n == 1]
-    tiles = [[i, q_starts[i], n] for i, n in enumerate(q_lens) if 1 < n <= 32]
-    long_tiles = [[i, q_starts[i] + f, min(128, n - f)] for i, n in enumerate(q_lens) if n > 32 for f in range(0, n, 128)]
+    tiles = [[i, q_starts[i] + f, min(64, n - f)] for i, n in enumerate(q_lens) if n > 1 for f in range(0, n, 64)]
     return P.StepContext(
         dtype=dtype, device=torch.device(DEV), num_tokens=len(positions), num_seqs=len(seq_ids),
         positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
@@ -46,8 +45,7 @@ def make_ctx(cache, dtype, seq_ids, q_lens):
         slots=torch.tensor(slots, dtype=torch.int32, device=DEV), cache=cache, seq_ids=list(seq_ids),
         q_starts=q_starts, q_lens=list(q_lens), past_lens=past, host_slots=slots,
         decode_tokens=torch.tensor(dec, dtype=torch.int32, device=DEV),
-        prefill_tiles=torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 3),
-        prefill_long_tiles=torch.tensor(long_tiles, dtype=torch.int32, device=DEV).view(-1, 3))
+        prefill_tiles=torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 3))
 
 
 # ------------------------------------------------------------------ built-in parts, one at a time
