@@ -245,27 +245,47 @@ __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_s
                                          const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                                          int max_splits, const int* __restrict__ dec_tok,
                                          const int* __restrict__ positions, int nh, int nkv, int window) {
+  // blockDim = (items rounded up to wavefronts, G): the splits are dealt out to G groups of threads,
+  // whose loads are all in flight together; group 0 then adds the groups' sums in group order.
+  extern __shared__ float s_merge[];  // [G - 1][items][6]: four sums, maximum, sum of weights
   constexpr int SPLIT = 64 * TPW;
   const int kvh = blockIdx.x;
   const int tok = dec_tok[blockIdx.y];
   const int pos = positions[tok];
   const int start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int s_first = start / SPLIT, nsplits = pos / SPLIT - s_first + 1;
-  const int g = nh / nkv;
-  const int item = threadIdx.x;  // (head in group, chunk of four features)
-  if (item >= g * (HD / 4)) return;
-  const int c = item / (HD / 4), d = (item % (HD / 4)) * 4;
+  const int g = nh / nkv, items = g * (HD / 4);
+  const int item = threadIdx.x, group = threadIdx.y, groups = blockDim.y;  // item: (head in group, four features)
+  const bool live = item < items;
+  const int c = live ? item / (HD / 4) : 0, d = (item % (HD / 4)) * 4;
   const int64_t slot0 = (((int64_t)blockIdx.y * nkv + kvh) * max_splits + s_first) * g + c;
   float m = NEG_BIG, l = 0.f;
   f32x4 a = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-  for (int sp = 0; sp < nsplits; ++sp) {  // consecutive splits are g slots apart
-    const int64_t slot = slot0 + (int64_t)sp * g;
-    const float ms = part_ml[slot * 2], ls = part_ml[slot * 2 + 1];
-    const f32x4 v = *reinterpret_cast<const f32x4*>(part_acc + slot * HD + d);
+  if (live) {
+#pragma unroll 8
+    for (int sp = group; sp < nsplits; sp += groups) {  // consecutive splits are g slots apart
+      const int64_t slot = slot0 + (int64_t)sp * g;
+      const float ms = part_ml[slot * 2], ls = part_ml[slot * 2 + 1];
+      const f32x4 v = *reinterpret_cast<const f32x4*>(part_acc + slot * HD + d);
+      const float m_new = fmaxf(m, ms);
+      const float f_old = exp2f(m - m_new), f = exp2f(ms - m_new);
+      a = a * f_old + v * f;
+      l = l * f_old + ls * f;
+      m = m_new;
+    }
+    if (group > 0) {
+      float* dst = s_merge + ((int64_t)(group - 1) * items + item) * 6;
+      dst[0] = a[0]; dst[1] = a[1]; dst[2] = a[2]; dst[3] = a[3]; dst[4] = m; dst[5] = l;
+    }
+  }
+  __syncthreads();
+  if (!live || group > 0) return;
+  for (int other = 1; other < groups; ++other) {
+    const float* src = s_merge + ((int64_t)(other - 1) * items + item) * 6;
+    const float ms = src[4], ls = src[5];
     const float m_new = fmaxf(m, ms);
     const float f_old = exp2f(m - m_new), f = exp2f(ms - m_new);
-    a = a * f_old + v * f;
+    a = a * f_old + (f32x4){src[0], src[1], src[2], src[3]} * f;
     l = l * f_old + ls * f;
     m = m_new;
   }
@@ -589,12 +609,21 @@ extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q
   const int max_splits = (int)(((int64_t)max_blocks * bs + split_len - 1) / split_len);
   const float scale_log2 = scale * LOG2E;
   dim3 grid(max_splits, nkv, num_dec), merge_grid(nkv, num_dec);
+  // merge: one thread per (head of the group, four features) and group of splits; up to four
+  // groups as far as 1,024 threads and the number of splits go
+  const int merge_items = nh / nkv * (hd / 4);
+  const int merge_x = (merge_items + PAE_WAVE - 1) / PAE_WAVE * PAE_WAVE;
+  int merge_groups = 1024 / merge_x < 4 ? 1024 / merge_x : 4;
+  if (merge_groups > max_splits) merge_groups = max_splits;
+  if (merge_groups < 1) merge_groups = 1;
+  PAE_REQUIRE(merge_x <= 1024, "attn_decode: %d heads of %d features per key/value head exceed the merge's workgroup", nh / nkv, hd);
+  const size_t merge_lds = (size_t)(merge_groups - 1) * merge_items * 6 * sizeof(float);
 #define CALL(HD)                                                                                            \
   attn_decode_kernel<HD, DECODE_TPW><<<grid, 256, (size_t)3 * (HD / 4 + 2) * PAE_WAVE * sizeof(float), stream>>>( \
       (float*)part_acc, (float*)part_ml, max_splits, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,     \
       (const bf16_t*)v_cache, dec_tok, positions, tok_seq, block_tables, max_blocks, bs, nh, nkv, scale_log2, \
       window);                                                                                               \
-  attn_decode_merge_kernel<HD, DECODE_TPW><<<merge_grid, (nh / nkv * (HD / 4) + 63) / 64 * 64, 0, stream>>>( \
+  attn_decode_merge_kernel<HD, DECODE_TPW><<<merge_grid, dim3(merge_x, merge_groups), merge_lds, stream>>>( \
       (bf16_t*)out, out_stride, (const float*)part_acc, (const float*)part_ml, max_splits, dec_tok, positions, \
       nh, nkv, window)
   FOR_HEAD_DIM(hd, CALL)
@@ -614,9 +643,8 @@ extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* 
   if (num_tiles <= 0) return 0;
   const float scale_log2 = scale * LOG2E;
   // four column tiles (64 tokens) per workgroup up to head_dim 128, two above (registers)
-#define SPLIT_CT 4
 #define LAUNCH(HD, BS)                                                                                         \
-  attn_prefill_split_kernel<HD, SPLIT_CT, BS><<<dim3(nh, num_tiles, 4 / SPLIT_CT), 256, 0, stream>>>( \
+  attn_prefill_split_kernel<HD, (HD <= 128 ? 4 : 2), BS><<<dim3(nh, num_tiles, HD <= 128 ? 1 : 2), 256, 0, stream>>>( \
       (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,    \
       tiles, positions, block_tables, max_blocks, bs, nh, nkv, scale_log2, window)
 #define CALL(HD)        \

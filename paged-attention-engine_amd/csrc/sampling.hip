@@ -106,31 +106,50 @@ __global__ __launch_bounds__(SAMPLE_NT) void sample_pick_kernel(int* __restrict_
   __shared__ double s_seg[SAMPLE_NT];
   __shared__ double s_before;
   __shared__ int s_where;
+  __shared__ float s_cmax[128];
+  __shared__ int s_carg[128];
+  __shared__ double s_csum[128];
   const int r = blockIdx.x, tid = threadIdx.x;
   const float temp = temperature ? temperature[r] : 0.f;
-  if (!(temp > 0.f)) {
-    if (tid == 0) {  // chunks in index order, strict comparison: the first maximum wins
-      float best = chunk_max[r * chunks];
-      int arg = chunk_arg[r * chunks];
-      for (int c = 1; c < chunks; ++c)
-        if (chunk_arg[r * chunks + c] >= 0 && (arg < 0 || chunk_max[r * chunks + c] > best)) {
-          best = chunk_max[r * chunks + c];
-          arg = chunk_arg[r * chunks + c];
-        }
-      tokens[r] = arg;
+  // the chunks' results come in with one load per thread; one thread then walks them in index order
+  if (tid < chunks) {
+    s_cmax[tid] = chunk_max[r * chunks + tid];
+    s_carg[tid] = chunk_arg[r * chunks + tid];
+    if (temp > 0.f) s_csum[tid] = chunk_sum[r * chunks + tid];
+  }
+  __syncthreads();
+  if (!(temp > 0.f)) {  // the same for the whole workgroup
+    // pairwise: the larger value wins, and among equal values the smaller index (the first maximum)
+    if (tid >= chunks && tid < 128) {
+      s_cmax[tid] = -INFINITY;
+      s_carg[tid] = -1;
     }
+    __syncthreads();
+    for (int step = 64; step > 0; step >>= 1) {
+      if (tid < step) {
+        const float ov = s_cmax[tid + step], mv = s_cmax[tid];
+        const int oi = s_carg[tid + step], mi = s_carg[tid];
+        if (oi >= 0 && (mi < 0 || ov > mv || (ov == mv && oi < mi))) {
+          s_cmax[tid] = ov;
+          s_carg[tid] = oi;
+        }
+      }
+      __syncthreads();
+    }
+    if (tid == 0) tokens[r] = s_carg[0];
     return;
   }
   const float* row = logits + (int64_t)r * ld;
-  const float row_max = row_maximum(chunk_max, r, chunks);
+  float row_max = s_cmax[0];
+  for (int c = 1; c < chunks; ++c) row_max = fmaxf(row_max, s_cmax[c]);
   if (tid == 0) {
     double total = 0.0;
-    for (int c = 0; c < chunks; ++c) total += chunk_sum[r * chunks + c];
+    for (int c = 0; c < chunks; ++c) total += s_csum[c];
     const double target = (double)uniform[r] * total;
     double run = 0.0;
     int where = -1;
     for (int c = 0; c < chunks; ++c) {
-      const double v = chunk_sum[r * chunks + c];
+      const double v = s_csum[c];
       if (run + v > target) { where = c; break; }
       run += v;
     }

@@ -416,6 +416,23 @@ def test_matrix_core_long_prefill_shapes(nh, nkv, hd, bs, window):
 
 
 # ------------------------------------------------------------------ sampling
+def test_argmax_ties_across_chunks():
+    """A vocabulary of many chunks, the maximum tied between chunks: the first index wins
+    (torch.argmax's rule, which the reference's greedy path relies on)."""
+    V = 70001
+    logits = torch.randn(5, V)
+    logits[0, [69000, 1500, 30000]] = 50.0
+    logits[1, [V - 1, V - 2]] = 50.0
+    logits[2, 0] = 50.0
+    logits[3, :] = 1.25           # everything tied
+    logits[4, [40000, 40001]] = 50.0
+    tokens = torch.empty(5, dtype=torch.int32, device=DEV)
+    K().sample(tokens, logits.to(DEV), None, None)
+    assert tokens.cpu().tolist() == [1500, V - 2, 0, 0, 40000]
+    K().sample(tokens, logits.to(DEV), torch.zeros(5, device=DEV), torch.rand(5, device=DEV))
+    assert tokens.cpu().tolist() == [1500, V - 2, 0, 0, 40000]
+
+
 def test_sampling_kernel():
     torch.manual_seed(5)
     V = 1000
