@@ -235,7 +235,7 @@ extern "C" int pae_residual_add(int dtype, void* residual, const void* delta, in
 // values transposed within the page, [block][kv head][hd][bs].
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, int nh, int nkv, int hd,
-                                     int rot, const float* __restrict__ inv_freq,
+                                     int rot, const float* __restrict__ cos_sin,
                                      const int* __restrict__ positions, const int* __restrict__ tok_seq,
                                      const int* __restrict__ block_tables, int max_blocks, int bs,
                                      T* __restrict__ k_cache, T* __restrict__ v_cache, int write_kv) {
@@ -254,8 +254,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, in
   const int rotated_heads = nh + (write_kv ? nkv : 0);
   for (int idx = threadIdx.x; idx < rotated_heads * half; idx += blockDim.x) {
     const int h = idx / half, i = idx % half;
-    float s = 0.f, c = 1.f;
-    if (inv_freq) sincosf((float)pos * inv_freq[i], &s, &c);
+    const float c = cos_sin[((int64_t)t * half + i) * 2], s = cos_sin[((int64_t)t * half + i) * 2 + 1];
     const float a = to_f32(row[h * hd + i]), b = to_f32(row[h * hd + i + half]);
     const T lo = from_f32<T>(a * c - b * s), hi = from_f32<T>(b * c + a * s);
     if (h < nh) {  // queries are rotated in place
@@ -280,23 +279,45 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, in
   }
 }
 
+// cos_sin[t][i] = (cos, sin)(positions[t] * inv_freq[i]) for i < half: computed once per step and
+// shared by every layer with the same rotation (angles in float32: engine/model.py:138-152).
+__global__ void rope_table_kernel(float* __restrict__ cos_sin, const int* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, int half, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  float s, c;
+  sincosf((float)positions[idx / half] * inv_freq[idx % half], &s, &c);
+  cos_sin[idx * 2] = c;
+  cos_sin[idx * 2 + 1] = s;
+}
+
+extern "C" int pae_rope_table(float* cos_sin, const int* positions, const float* inv_freq, int num_tokens, int half,
+                              hipStream_t stream) {
+  PAE_REQUIRE(num_tokens >= 0 && half > 0, "rope_table: bad sizes T=%d half=%d", num_tokens, half);
+  const int64_t total = (int64_t)num_tokens * half;
+  if (total == 0) return 0;
+  rope_table_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(cos_sin, positions, inv_freq, half, total);
+  return pae_check_launch("rope_table");
+}
+
 extern "C" int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv,
-                                 int hd, int rot, const float* inv_freq, const int* positions,
+                                 int hd, int rot, const float* cos_sin, const int* positions,
                                  const int* tok_seq, const int* block_tables, int max_blocks, int bs,
                                  void* k_cache, void* v_cache, int write_kv, hipStream_t stream) {
   PAE_REQUIRE(nh > 0 && nkv >= 0 && hd > 0, "rope_kv_write: bad head sizes nh=%d nkv=%d hd=%d", nh, nkv, hd);
   PAE_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rot, hd);
+  PAE_REQUIRE(rot == 0 || cos_sin, "rope_kv_write: a rotation needs its table of cosines and sines");
   PAE_REQUIRE(row_stride >= (int64_t)(nh + 2 * nkv) * hd, "rope_kv_write: row stride %lld too small", (long long)row_stride);
   PAE_REQUIRE(!write_kv || (bs > 0 && max_blocks > 0 && k_cache && v_cache && block_tables && tok_seq),
               "rope_kv_write: cache write needs tables and pools");
   if (num_tokens <= 0) return 0;
   if (dtype == PAE_F32)
     rope_kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>(
-        (float*)qkv, row_stride, nh, nkv, hd, rot, inv_freq, positions, tok_seq, block_tables, max_blocks, bs,
+        (float*)qkv, row_stride, nh, nkv, hd, rot, cos_sin, positions, tok_seq, block_tables, max_blocks, bs,
         (float*)k_cache, (float*)v_cache, write_kv);
   else if (dtype == PAE_BF16)
     rope_kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
-        (bf16_t*)qkv, row_stride, nh, nkv, hd, rot, inv_freq, positions, tok_seq, block_tables, max_blocks, bs,
+        (bf16_t*)qkv, row_stride, nh, nkv, hd, rot, cos_sin, positions, tok_seq, block_tables, max_blocks, bs,
         (bf16_t*)k_cache, (bf16_t*)v_cache, write_kv);
   else
     return pae_fail("rope_kv_write: unknown dtype code %d", dtype);

@@ -33,7 +33,7 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 // What the rotating epilogue needs beside the product: the head geometry, the
 // rotation's frequencies, every row's position and sequence, and the paged cache.
 struct SkinnyRope {
-  const float* inv_freq;    // [rot / 2], or null without rotation
+  const float* cos_sin;     // [M][rot / 2][2] cosine and sine of every row's angles, or null without rotation
   const int* positions;     // [M]
   const int* tok_seq;       // [M] row of block_tables
   const int* block_tables;  // [sequences][max_blocks]
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
                                                           int N, int K, int k_per_split, int64_t part_stride,
                                                           SkinnyRope rope) {
   static_assert(EPI != EPI_SWIGLU || RT % 2 == 0, "the gated epilogue pairs a gate tile with its up tile");
-  __shared__ float s_part[3][RT * MT * 4][PAE_WAVE];
+  __shared__ float s_part[MT == 1 ? 3 : 4][RT * MT * 4][PAE_WAVE];
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
   const int n0 = blockIdx.x * 16 * RT;
@@ -144,24 +144,46 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
     }
   }
 
-  if (wave > 0) {
+  // The four wavefronts' sums are added in wavefront order.  With one column tile wavefront 0 adds
+  // and writes; with more, wavefront w takes column tile w, so that the epilogues run side by side.
+  if (MT == 1) {
+    if (wave > 0) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_part[wave - 1][rt * 4 + i][lane] = acc[rt][0][i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[rt][0][i] += s_part[w][rt * 4 + i][lane];
+  } else {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) s_part[wave - 1][(rt * MT + mt) * 4 + i][lane] = acc[rt][mt][i];
+        for (int i = 0; i < 4; ++i) s_part[wave][(rt * MT + mt) * 4 + i][lane] = acc[rt][mt][i];
+    __syncthreads();
+    if (wave >= MT) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      if (mt == wave) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float sum = s_part[0][(rt * MT + mt) * 4 + i][lane];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) sum += s_part[w][(rt * MT + mt) * 4 + i][lane];
+            acc[rt][mt][i] = sum;
+          }
+      }
   }
-  __syncthreads();
-  if (wave > 0) return;
-#pragma unroll
-  for (int w = 0; w < 3; ++w)
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[rt][mt][i] += s_part[w][(rt * MT + mt) * 4 + i][lane];
 
   if (EPI == EPI_ROPE) {
     // lane holds row m = 16 mt + r of A and rows 4 g4 + i of each tile: lanes 0-31 the lower
@@ -170,6 +192,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
     const int64_t head_step = (int64_t)rope.bs * rope.hd;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
+      if (MT > 1 && mt != wave) continue;  // another wavefront's column tile
       const int m = 16 * mt + r;
       const int mc = m < M ? m : M - 1;
       const int pos = rope.positions[mc];
@@ -189,8 +212,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
           const float other = __shfl_xor(own, 32);  // in every lane
           float o = own;
           if (rotated) {
-            float sn, cs;
-            sincosf((float)pos * rope.inv_freq[8 * j + (4 * g4 + i) % 8], &sn, &cs);
+            const float* angle = rope.cos_sin + ((int64_t)mc * (rope.rot / 2) + 8 * j + (4 * g4 + i) % 8) * 2;
+            const float cs = angle[0], sn = angle[1];
             o = g4 < 2 ? own * cs - other * sn : own * cs + other * sn;
           }
           res[i] = to_bf16_bits(o);
@@ -220,6 +243,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
   // lane holds, per column tile mt, row m = 16 mt + r of A and weight rows 4 g4 + i of each row tile
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
+    if (MT > 1 && mt != wave) continue;  // another wavefront's column tile
     const int m = 16 * mt + r;
     if (m >= M) continue;
     if (EPI == EPI_SWIGLU) {
@@ -318,20 +342,21 @@ extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void*
 // q_out[M, nh * hd] = rotated queries of A * W^T (+ bias), W = [(nh + 2 nkv) * hd, K] holding the
 // query, key and value projections in that order; rotated keys and raw values of every row go to
 // slot block_tables[tok_seq[m]][positions[m] / bs] * bs + positions[m] % bs of the cache.  With
-// nkv == 0 only queries are projected and nothing is stored.  rot == 0 (inv_freq null) rotates nothing.
+// nkv == 0 only queries are projected and nothing is stored.  rot == 0 (cos_sin null) rotates nothing;
+// else cos_sin[m][i] = (cos, sin) of row m's angle for pair i < rot / 2.
 extern "C" int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int64_t lda, const void* W,
                                     const void* bias, int b_is_f32, int M, int K, int nh, int nkv, int hd, int rot,
-                                    const float* inv_freq, const int* positions, const int* tok_seq,
+                                    const float* cos_sin, const int* positions, const int* tok_seq,
                                     const int* block_tables, int max_blocks, int bs, void* k_cache, void* v_cache,
                                     hipStream_t stream) {
   PAE_REQUIRE(nh > 0 && nkv >= 0 && hd > 0 && hd % 16 == 0, "gemm_skinny_rope: bad head sizes nh=%d nkv=%d hd=%d", nh, nkv, hd);
-  PAE_REQUIRE(rot >= 0 && rot <= hd && rot % 16 == 0 && (rot == 0 || inv_freq),
+  PAE_REQUIRE(rot >= 0 && rot <= hd && rot % 16 == 0 && (rot == 0 || cos_sin),
               "gemm_skinny_rope: rotary_dim %d must be a multiple of 16 up to head_dim %d", rot, hd);
   PAE_REQUIRE(ldq >= (int64_t)nh * hd && ldq % 4 == 0, "gemm_skinny_rope: row stride %lld of the queries", (long long)ldq);
   PAE_REQUIRE(positions, "gemm_skinny_rope: positions are missing");
   PAE_REQUIRE(nkv == 0 || (bs > 0 && max_blocks > 0 && k_cache && v_cache && block_tables && tok_seq),
               "gemm_skinny_rope: the cache write needs tables and pools");
-  SkinnyRope rope{inv_freq, positions, tok_seq, block_tables, (bf16_t*)k_cache, (bf16_t*)v_cache,
+  SkinnyRope rope{cos_sin, positions, tok_seq, block_tables, (bf16_t*)k_cache, (bf16_t*)v_cache,
                   nh, nkv, hd, rot, max_blocks, bs};
   return launch_skinny(EPI_ROPE, q_out, ldq, A, lda, W, bias, b_is_f32, M, (nh + 2 * nkv) * hd, K, 1, 0, rope, stream);
 }

@@ -54,6 +54,7 @@ def _declare(lib) -> None:
         "pae_embedding": [I, P, P, P, I, I, I, P],
         "pae_add_rmsnorm": [I, P, P, I, L, P, I, F, P, P, I, I, I, P],
         "pae_residual_add": [I, P, P, L, P],
+        "pae_rope_table": [P, P, P, I, I, P],
         "pae_rope_kv_write": [I, P, L, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P],
         "pae_swiglu": [I, P, P, I, I, I, P],
         "pae_gemm_skinny": [I, P, L, P, L, P, P, I, I, I, I, I, L, P],
@@ -169,18 +170,34 @@ def residual_add(residual: torch.Tensor, delta: torch.Tensor) -> None:
                                       residual.numel(), _stream()))
 
 
-def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, inv_freq: Optional[torch.Tensor],
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """[T, len(inv_freq), 2] float32: cosine and sine of positions[t] * inv_freq[i]."""
+    _gpu(positions, inv_freq)
+    assert positions.dtype == torch.int32 and inv_freq.dtype == torch.float32 and inv_freq.is_contiguous()
+    T, half = positions.numel(), inv_freq.numel()
+    out = torch.empty((T, half, 2), dtype=torch.float32, device=positions.device)
+    _check(library().pae_rope_table(out.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(), T, half, _stream()))
+    return out
+
+
+def _check_cos_sin(cos_sin: Optional[torch.Tensor], rot: int, T: int) -> None:
+    if rot:
+        assert cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
+        assert tuple(cos_sin.shape) == (T, rot // 2, 2)
+
+
+def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, cos_sin: Optional[torch.Tensor],
                   positions: torch.Tensor, tok_seq: Optional[torch.Tensor], block_tables: Optional[torch.Tensor],
                   block_size: int, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor]) -> None:
-    """Rotate the query heads of `qkv` in place; rotate the key heads and copy the
-    value heads into their cache slots (skipped when `k_cache` is None: then the
-    row holds query heads only and nkv must be 0)."""
-    _gpu(qkv, inv_freq, positions, tok_seq, block_tables, k_cache, v_cache)
+    """Rotate the query heads of `qkv` in place by the angles whose cosines and sines `cos_sin`
+    holds ([T, rot / 2, 2], see `rope_table`); rotate the key heads and copy the value heads
+    into their cache slots (skipped when `k_cache` is None: then the row holds query heads only
+    and nkv must be 0)."""
+    _gpu(qkv, cos_sin, positions, tok_seq, block_tables, k_cache, v_cache)
     T = qkv.shape[0]
     assert qkv.dim() == 2 and qkv.stride(1) == 1 and positions.dtype == torch.int32 and positions.numel() == T
     write = k_cache is not None
-    if inv_freq is not None:
-        assert inv_freq.dtype == torch.float32 and inv_freq.numel() == rot // 2
+    _check_cos_sin(cos_sin, rot, T)
     max_blocks = 0
     if write:
         assert v_cache is not None and k_cache.dtype == qkv.dtype == v_cache.dtype
@@ -189,9 +206,9 @@ def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, inv_f
         _check_pools(k_cache, v_cache, nkv, block_size, hd)
         max_blocks = block_tables.shape[1]
     _check(library().pae_rope_kv_write(code_of(qkv.dtype), qkv.data_ptr(), qkv.stride(0), T, nh, nkv, hd, rot,
-                                       _ptr(inv_freq), positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables),
-                                       max_blocks, block_size, _ptr(k_cache), _ptr(v_cache), 1 if write else 0,
-                                       _stream()))
+                                       _ptr(cos_sin) if rot else None, positions.data_ptr(), _ptr(tok_seq),
+                                       _ptr(block_tables), max_blocks, block_size, _ptr(k_cache), _ptr(v_cache),
+                                       1 if write else 0, _stream()))
 
 
 def swiglu(out: torch.Tensor, x: torch.Tensor, block: int = 0) -> None:
@@ -253,19 +270,18 @@ def skinny_rope_supported(a: torch.Tensor, w: torch.Tensor, hd: int, rot: int) -
 
 
 def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], nh: int,
-                     nkv: int, hd: int, rot: int, inv_freq: Optional[torch.Tensor], positions: torch.Tensor,
+                     nkv: int, hd: int, rot: int, cos_sin: Optional[torch.Tensor], positions: torch.Tensor,
                      tok_seq: Optional[torch.Tensor], block_tables: Optional[torch.Tensor], block_size: int,
                      k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor]) -> None:
     """Query/key/value projection of at most 64 rows with the rotation and the cache write in its
     epilogue: q_out[M, nh * hd] = rotated queries; rotated keys and raw values go to their slots
-    (nkv == 0: `w` holds the query rows only and nothing is stored)."""
-    _gpu(q_out, a, w, bias, inv_freq, positions, tok_seq, block_tables, k_cache, v_cache)
+    (nkv == 0: `w` holds the query rows only and nothing is stored).  `cos_sin`: see `rope_table`."""
+    _gpu(q_out, a, w, bias, cos_sin, positions, tok_seq, block_tables, k_cache, v_cache)
     M, K_ = a.shape
     assert skinny_rope_supported(a, w, hd, rot) and w.shape == ((nh + 2 * nkv) * hd, K_) and w.is_contiguous()
     assert q_out.shape == (M, nh * hd) and q_out.dtype == torch.bfloat16 and q_out.stride(1) == 1
     assert positions.dtype == torch.int32 and positions.numel() == M
-    if rot:
-        assert inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() == rot // 2
+    _check_cos_sin(cos_sin, rot, M)
     max_blocks = 0
     if nkv:
         assert k_cache.dtype == torch.bfloat16 == v_cache.dtype
@@ -275,7 +291,7 @@ def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias
         max_blocks = block_tables.shape[1]
     bp, bf = _param(bias)
     _check(library().pae_gemm_skinny_rope(q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(),
-                                          bp, bf, M, K_, nh, nkv, hd, rot, _ptr(inv_freq) if rot else None,
+                                          bp, bf, M, K_, nh, nkv, hd, rot, _ptr(cos_sin) if rot else None,
                                           positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks,
                                           block_size, _ptr(k_cache), _ptr(v_cache), _stream()))
 

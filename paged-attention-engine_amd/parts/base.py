@@ -54,15 +54,17 @@ class StepContext:
     q_lens: List[int] = field(default_factory=list)     # rows of each sequence in this step
     past_lens: List[int] = field(default_factory=list)  # tokens each sequence held before the step
     host_slots: List[int] = field(default_factory=list)
-    # work lists of the attention kernels: sequences that bring one token; runs of up to 32
-    # consecutive tokens of sequences that bring 2..32, and runs of up to 128 of those that
-    # bring more, each as (table row, first flat token, count)
+    # work lists of the attention kernels: sequences that bring one token, and runs of up to 64
+    # consecutive tokens of the others as (table row, first flat token, count), most keys first
     decode_tokens: Optional[torch.Tensor] = None   # int32 [number of single-token sequences]
     prefill_tiles: Optional[torch.Tensor] = None   # int32 [runs of 2..64 tokens, 3]: table row, first token, count
     # set by the model for the stop that is running
     entry: int = 0                     # index in the schedule
     cache_entry: int = 0               # the stop whose cache is read (entry itself unless it borrows)
     writes_cache: bool = True
+    # what a part computes once per step for every layer that has the same part (a table of angles,
+    # say), under a key of the part's choosing
+    memo: Dict[object, object] = field(default_factory=dict)
 
 
 class Part:

@@ -27,25 +27,35 @@ class NeoxRope(Part):
         exponent = torch.arange(0, rot, 2, dtype=torch.int64).to(torch.float32)
         self.inv_freq = (1.0 / (spec.theta ** (exponent / rot))).to(device)
 
+    def cos_sin(self, ctx):
+        """Cosines and sines of every token's angles, computed by the first layer of a step that
+        asks and shared by all layers with the same rotation."""
+        if not self.spec.rotary_dim:
+            return None
+        key = ("neox_rope", self.spec.rotary_dim, self.spec.theta)
+        table = ctx.memo.get(key)
+        if table is None:
+            table = ctx.memo[key] = K.rope_table(ctx.positions, self.inv_freq)
+        return table
+
     def encode_and_store(self, ctx, qkv, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
         """Rotate the query heads of `qkv` in place; write rotated keys and raw
         values to the cache (when `k_cache` is given)."""
-        K.rope_kv_write(qkv, nh, nkv, hd, self.spec.rotary_dim, self.inv_freq, ctx.positions, ctx.tok_seq,
+        K.rope_kv_write(qkv, nh, nkv, hd, self.spec.rotary_dim, self.cos_sin(ctx), ctx.positions, ctx.tok_seq,
                         block_table, block_size, k_cache, v_cache)
-
 
     def project_encode_store(self, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
         """The projection, the rotation and the cache write as one kernel, where there is one for
         these sizes; otherwise None, and the caller runs the two steps."""
-        return _fused_projection(self.spec.rotary_dim, self.inv_freq, ctx, x, linear, nh, nkv, hd, k_cache,
+        if x.dtype != torch.bfloat16 or not K.skinny_rope_supported(x, linear.weight, hd, self.spec.rotary_dim):
+            return None
+        return _fused_projection(self.spec.rotary_dim, self.cos_sin(ctx), ctx, x, linear, nh, nkv, hd, k_cache,
                                  v_cache, block_table, block_size)
 
 
-def _fused_projection(rot, inv_freq, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
-    if x.dtype != torch.bfloat16 or not K.skinny_rope_supported(x, linear.weight, hd, rot):
-        return None
+def _fused_projection(rot, cos_sin, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
     q = torch.empty((x.shape[0], nh * hd), dtype=x.dtype, device=x.device)
-    K.gemm_skinny_rope(q, x, linear.weight, linear.bias, nh, nkv, hd, rot, inv_freq, ctx.positions, ctx.tok_seq,
+    K.gemm_skinny_rope(q, x, linear.weight, linear.bias, nh, nkv, hd, rot, cos_sin, ctx.positions, ctx.tok_seq,
                        block_table, block_size, k_cache, v_cache)
     return q
 
@@ -61,4 +71,6 @@ class NoPosition(Part):
                             k_cache, v_cache)
 
     def project_encode_store(self, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
+        if x.dtype != torch.bfloat16 or not K.skinny_rope_supported(x, linear.weight, hd, 0):
+            return None
         return _fused_projection(0, None, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size)

@@ -209,6 +209,17 @@ def reference_attention(q, k, v, pos, scale, window):
 
 
 # ------------------------------------------------------------------ rotation and cache write
+def test_rope_table():
+    """Angles are position * inv_freq in float32 (engine/model.py:138-152 of the reference)."""
+    positions = torch.tensor([0, 1, 2, 77, 4095, 32767, 131071], dtype=torch.int32)
+    inv = plain.rope_inv_freq(48, 1e6)
+    got = K().rope_table(positions.to(DEV), inv.to(DEV)).cpu()
+    angle = (positions.float()[:, None] * inv[None, :]).double()  # the float32 product, as the reference forms it
+    assert got.shape == (7, 24, 2)
+    assert (got[..., 0].double() - angle.cos()).abs().max() <= 2e-6
+    assert (got[..., 1].double() - angle.sin()).abs().max() <= 2e-6
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nh,nkv,hd,rot,bs", [(4, 2, 16, 16, 4), (6, 1, 48, 48, 16), (3, 3, 32, 16, 8)])
 def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs):
@@ -220,11 +231,12 @@ def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs):
     tables = scattered_tables([12, 38], bs, 40, seed=3)
     T = len(positions)
     qkv = torch.randn(T, (nh + 2 * nkv) * hd).to(DT[dtype])
-    inv = plain.rope_inv_freq(rot, theta)
+    pos_d = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    table = K().rope_table(pos_d, plain.rope_inv_freq(rot, theta).to(DEV))
     kp = torch.full((40, nkv, bs, hd), 7.0, dtype=DT[dtype])
     vp = torch.full((40, nkv, hd, bs), 7.0, dtype=DT[dtype])
     d_qkv, d_kp, d_vp = qkv.to(DEV), kp.to(DEV), vp.to(DEV)
-    K().rope_kv_write(d_qkv, nh, nkv, hd, rot, inv.to(DEV), torch.tensor(positions, dtype=torch.int32, device=DEV),
+    K().rope_kv_write(d_qkv, nh, nkv, hd, rot, table, pos_d,
                       torch.tensor(tok_seq, dtype=torch.int32, device=DEV), tables.to(DEV), bs, d_kp, d_vp)
     x = qkv.double().view(T, nh + 2 * nkv, hd)
     cos, sin = plain.rope_cos_sin(plain.rope_inv_freq(rot, theta, torch.float64), torch.tensor(positions), torch.float64)
@@ -270,7 +282,8 @@ def test_gemm_skinny_rope(M, nh, nkv, hd, rot, bs, Kdim, bias):
     vp = torch.full((num_blocks, nkv, hd, bs), 7.0, dtype=torch.bfloat16)
     d_kp, d_vp = kp.to(DEV), vp.to(DEV)
     q = torch.full((M, nh * hd), 9.0, dtype=torch.bfloat16, device=DEV)
-    inv = plain.rope_inv_freq(rot, theta).to(DEV) if rot else None
+    inv = (K().rope_table(torch.tensor(positions, dtype=torch.int32, device=DEV), plain.rope_inv_freq(rot, theta).to(DEV))
+           if rot else None)
     K().gemm_skinny_rope(q, a.to(DEV), w.to(DEV), None if b is None else b.to(DEV), nh, nkv, hd, rot, inv,
                          torch.tensor(positions, dtype=torch.int32, device=DEV),
                          torch.tensor(tok_seq, dtype=torch.int32, device=DEV), tables.to(DEV), bs, d_kp, d_vp)
