@@ -115,32 +115,59 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
   // addresses, and issued SKINNY_U steps ahead of their use; a lane past the end of
   // the k range zeroes its weight fragment (rows past N or M are simply not stored).
   const bf16x8 zero = {};
-  for (int kb = k_lo + 32 * wave; kb < k_hi; kb += 128 * SKINNY_U) {
+  struct Batch {  // SKINNY_U steps of a wavefront: k offsets kb + 128 u
     bf16x8 wf[SKINNY_U][RT], af[SKINNY_U][MT];
+  };
+  auto load = [&](Batch& b, int kb) {
 #pragma unroll
     for (int u = 0; u < SKINNY_U; ++u) {
       const int k = kb + 128 * u + 8 * lkg;
       const int kc = k < K - 8 ? k : K - 8;
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) wf[u][rt] = *reinterpret_cast<const bf16x8*>(wrow[rt] + kc);
+      for (int rt = 0; rt < RT; ++rt) b.wf[u][rt] = *reinterpret_cast<const bf16x8*>(wrow[rt] + kc);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) af[u][mt] = *reinterpret_cast<const bf16x8*>(arow[mt] + kc);
+      for (int mt = 0; mt < MT; ++mt) b.af[u][mt] = *reinterpret_cast<const bf16x8*>(arow[mt] + kc);
     }
+  };
+  auto multiply = [&](Batch& b, int kb) {
 #pragma unroll
     for (int u = 0; u < SKINNY_U; ++u) {
       // K and the range bounds are multiples of 8: a lane's 8 elements are all in or all out
       const bool kok = kb + 128 * u + 8 * g4 < k_hi;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) af[u][mt] = to_mfma_order(af[u][mt], fetch_from);
+      for (int mt = 0; mt < MT; ++mt) b.af[u][mt] = to_mfma_order(b.af[u][mt], fetch_from);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         // the permute runs in every lane (a lane that skipped it could not be read by the others)
-        const bf16x8 moved = to_mfma_order(wf[u][rt], fetch_from);
+        const bf16x8 moved = to_mfma_order(b.wf[u][rt], fetch_from);
         const bf16x8 w = kok ? moved : zero;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, af[u][mt], acc[rt][mt], 0, 0, 0);
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, b.af[u][mt], acc[rt][mt], 0, 0, 0);
       }
+    }
+  };
+  constexpr int STEP = 128 * SKINNY_U;
+  int kb = k_lo + 32 * wave;  // the same in every lane of a wavefront: the branches on it are uniform
+  if (MT == 1) {
+    // two batches take turns, so that a wavefront always has loads in flight: with one, every
+    // batch waits out the memory's latency before the next is even asked for
+    Batch b0, b1;
+    if (kb < k_hi) load(b0, kb);
+    while (kb < k_hi) {
+      if (kb + STEP < k_hi) load(b1, kb + STEP);
+      multiply(b0, kb);
+      kb += STEP;
+      if (kb >= k_hi) break;
+      if (kb + STEP < k_hi) load(b0, kb + STEP);
+      multiply(b1, kb);
+      kb += STEP;
+    }
+  } else {  // more column tiles: the registers go to the activations' fragments
+    for (; kb < k_hi; kb += STEP) {
+      Batch b;
+      load(b, kb);
+      multiply(b, kb);
     }
   }
 

@@ -203,6 +203,7 @@ class Scheduler:
         self._next_arrival = 0
         self._next_seq_id = 0
         self._pending: List[ScheduledWork] = []
+        self._pending_tokens = 0
 
     # ------------------------------------------------------------------ event log
     def _tokens_held(self) -> int:
@@ -240,7 +241,7 @@ class Scheduler:
 
     # ------------------------------------------------------------------ budget
     def _tokens_planned(self) -> int:
-        return sum(len(w.token_ids) for w in self._pending)
+        return self._pending_tokens  # kept beside `_pending` by `_plan`, `_evict` and `step`
 
     def _budget_left(self) -> int:
         """Tokens this step may still take; an empty batch may always take one."""
@@ -260,10 +261,12 @@ class Scheduler:
         self._pending.append(ScheduledWork(
             seq=seq, token_ids=tuple(history[start:end]), positions=tuple(range(start, end)),
             is_prefill=seq.prefilling, samples=end == len(history)))
+        self._pending_tokens += count
 
     def _evict(self, seq: Sequence) -> None:
         self.running.remove(seq)
         self._pending = [w for w in self._pending if w.seq is not seq]
+        self._pending_tokens = sum(len(w.token_ids) for w in self._pending)
         freed = self.cache.free_sequence(seq.seq_id)
         seq.seq_id = None
         seq.num_computed = 0
@@ -321,6 +324,7 @@ class Scheduler:
     def step(self) -> StepResult:
         self._step += 1
         self._pending = []
+        self._pending_tokens = 0
         preempted: List[str] = []
         deferred: List[str] = []
         admitted: List[Sequence] = []
@@ -365,7 +369,7 @@ class Scheduler:
         # 3. one pass of the model for everything planned
         batch = self._pending
         self._pending = []
-        tokens_run = sum(len(w.token_ids) for w in batch)
+        tokens_run, self._pending_tokens = self._pending_tokens, 0
         if batch:
             results = self.executor.execute(batch, self.record_logits)
             if len(results) != len(batch):
