@@ -125,6 +125,16 @@ class Sequence:
     def history_len(self) -> int:
         return self.request.prompt_len + len(self.generated)
 
+    def history_slice(self, start: int, end: int) -> Tuple[int, ...]:
+        """history[start:end] without building the whole history (a decode step asks for one token)."""
+        prompt = self.request.prompt_token_ids
+        n = len(prompt)
+        if start >= n:
+            return tuple(self.generated[start - n:end - n])
+        if end <= n:
+            return tuple(prompt[start:end])
+        return tuple(prompt[start:]) + tuple(self.generated[:end - n])
+
     @property
     def is_finished(self) -> bool:
         return self.stopped or len(self.generated) >= self.request.max_new_tokens
@@ -255,12 +265,11 @@ class Scheduler:
         result = self.cache.reserve(seq.seq_id, count)
         if not result.ok:
             raise AssertionError(f"{seq.request_id}: reserving {count} token(s) failed after the capacity check")
-        history = seq.history
         start = seq.num_computed
         end = start + count
         self._pending.append(ScheduledWork(
-            seq=seq, token_ids=tuple(history[start:end]), positions=tuple(range(start, end)),
-            is_prefill=seq.prefilling, samples=end == len(history)))
+            seq=seq, token_ids=seq.history_slice(start, end), positions=tuple(range(start, end)),
+            is_prefill=seq.prefilling, samples=end == seq.history_len))
         self._pending_tokens += count
 
     def _evict(self, seq: Sequence) -> None:

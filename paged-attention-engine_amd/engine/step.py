@@ -13,6 +13,8 @@ reserved room for every token (:414-417), so positions are the run
 
 from __future__ import annotations
 
+from array import array
+
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -128,7 +130,7 @@ class StepRunner:
             for table in per_seq:
                 flat.extend(table)
                 flat.extend([-1] * (width - len(table)))
-        staging = torch.tensor(flat, dtype=torch.int32).pin_memory()
+        staging = torch.frombuffer(array("i", flat), dtype=torch.int32).pin_memory()
 
         captured = None
         if decode_only:

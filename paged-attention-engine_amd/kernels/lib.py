@@ -79,7 +79,8 @@ def _check(code: int) -> None:
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    # the raw handle of torch's current stream (also the capture stream while a graph records)
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 def code_of(dtype: torch.dtype) -> int:
