@@ -148,8 +148,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
     }
   };
   constexpr int STEP = 128 * SKINNY_U;
+  constexpr bool PIPELINED = true;
   int kb = k_lo + 32 * wave;  // the same in every lane of a wavefront: the branches on it are uniform
-  if (MT == 1) {
+  if (PIPELINED) {
     // two batches take turns, so that a wavefront always has loads in flight: with one, every
     // batch waits out the memory's latency before the next is even asked for
     Batch b0, b1;
@@ -337,7 +338,7 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   dim3 grid((N + 16 * rt - 1) / (16 * rt), splits);
   // four k steps of loads in flight per wavefront: deeper prefetch costs registers and measured slower
 #define LAUNCH(MT, RT, EPI)                                                                                  \
-  gemm_skinny_kernel<MT, RT, EPI, 4><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
+  gemm_skinny_kernel<MT, RT, EPI, (MT == 1 ? 4 : 2)><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
                                                                bias, b_is_f32, M, N, K, k_per_split, part_stride, rope)
 #define BY_MT(EPI)                                                   \
   switch (mt) {                                                      \
