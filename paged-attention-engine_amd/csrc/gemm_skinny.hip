@@ -63,6 +63,120 @@ __device__ __forceinline__ short to_bf16_bits(float x) {
   return *reinterpret_cast<const short*>(&h);
 }
 
+// What a wavefront does with finished sums: acc[rt][mt] is the 16 x 16 tile of weight rows
+// 16 (tile_base + rt) .. (through the rotation's row order, if any) by rows 16 mt .. of A; a lane
+// holds row m = 16 mt + lane % 16 of A and weight rows 4 (lane / 16) + i.  only_mt >= 0: just
+// that column tile (the others belong to other wavefronts).
+template <int MT, int RT, int EPI>
+__device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int tile_base, int only_mt,
+                                                void* __restrict__ out, int64_t ldc, const void* __restrict__ bias,
+                                                int b_is_f32, int M, int N, int split, int64_t part_stride,
+                                                const SkinnyRope& rope) {
+  const int lane = threadIdx.x % PAE_WAVE;
+  const int r = lane % 16, g4 = lane / 16;
+  if (EPI == EPI_ROPE) {
+    // lane holds row m = 16 mt + r of A and rows 4 g4 + i of each tile: lanes 0-31 the lower
+    // features of the pairs, lanes 32-63 (same m) their partners
+    const int per_head = rope.hd / 16;
+    const int64_t head_step = (int64_t)rope.bs * rope.hd;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      if (only_mt >= 0 && mt != only_mt) continue;  // another wavefront's column tile
+      const int m = 16 * mt + r;
+      const int mc = m < M ? m : M - 1;
+      const int pos = rope.positions[mc];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int tile = tile_base + rt;
+        const int head = tile / per_head, j = tile % per_head;
+        const bool rotated = 16 * j < rope.rot && head < rope.nh + rope.nkv;  // values keep the tile layout, unrotated
+        const int f0 = rope_feature(j, 4 * g4, rope.rot);  // first of this lane's 4 consecutive features
+        const int n = head * rope.hd + f0;
+        s16x4 res;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          // the projection is rounded to bfloat16 before the rotation, as where the two are separate kernels
+          const float own = __bfloat162float(__float2bfloat16(
+              acc[rt][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f)));
+          const float other = __shfl_xor(own, 32);  // in every lane
+          float o = own;
+          if (rotated) {
+            const float* angle = rope.cos_sin + ((int64_t)mc * (rope.rot / 2) + 8 * j + (4 * g4 + i) % 8) * 2;
+            const float cs = angle[0], sn = angle[1];
+            o = g4 < 2 ? own * cs - other * sn : own * cs + other * sn;
+          }
+          res[i] = to_bf16_bits(o);
+        }
+        if (m >= M || n >= N) continue;
+        if (head < rope.nh) {
+          *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + n) = res;
+          continue;
+        }
+        const int off = pos % rope.bs;
+        const int64_t page = (int64_t)rope.block_tables[(int64_t)rope.tok_seq[m] * rope.max_blocks + pos / rope.bs] *
+                             rope.nkv * head_step;
+        if (head < rope.nh + rope.nkv) {
+          *reinterpret_cast<s16x4*>(rope.k_cache + page + (head - rope.nh) * head_step + (int64_t)off * rope.hd + f0) = res;
+        } else {
+          short* dst = reinterpret_cast<short*>(rope.v_cache) + page + (head - rope.nh - rope.nkv) * head_step +
+                       (int64_t)f0 * rope.bs + off;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[(int64_t)i * rope.bs] = res[i];
+        }
+      }
+    }
+    return;
+  }
+
+  const bool vec = ldc % 4 == 0;  // rows of out keep 8- and 16-byte stores aligned
+  // lane holds, per column tile mt, row m = 16 mt + r of A and weight rows 4 g4 + i of each row tile
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    if (only_mt >= 0 && mt != only_mt) continue;  // another wavefront's column tile
+    const int m = 16 * mt + r;
+    if (m >= M) continue;
+    if (EPI == EPI_SWIGLU) {
+#pragma unroll
+      for (int pair = 0; pair < RT / 2; ++pair) {  // tiles 2 pair (gate) and 2 pair + 1 (up)
+        const int j = (tile_base / 2 + pair) * 16 + 4 * g4;  // output feature of register 0
+        if (j >= N / 2) continue;                                    // N counts gate and up rows
+        s16x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float g = acc[2 * pair][mt][i], u = acc[2 * pair + 1][mt][i];
+          v[i] = to_bf16_bits(g / (1.0f + expf(-g)) * u);
+        }
+        *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j) = v;
+      }
+    } else {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int n = 16 * (tile_base + rt) + 4 * g4;
+        if (n >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          v[i] = acc[rt][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f);
+        if (EPI == EPI_F32) {
+          float* dst = (float*)out + (int64_t)split * part_stride + (int64_t)m * ldc + n;
+          if (vec && n + 4 <= N) *reinterpret_cast<f32x4*>(dst) = (f32x4){v[0], v[1], v[2], v[3]};
+          else
+            for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = v[i];
+        } else {
+          bf16_t* dst = (bf16_t*)out + (int64_t)m * ldc + n;
+          if (vec && n + 4 <= N) {
+            s16x4 p;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p[i] = to_bf16_bits(v[i]);
+            *reinterpret_cast<s16x4*>(dst) = p;
+          } else
+            for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = __float2bfloat16(v[i]);
+        }
+      }
+    }
+  }
+}
+
 // MT: column tiles of 16 rows of A; RT: tiles of 16 weight rows per workgroup; SKINNY_U: k steps
 // of a wavefront whose loads are in flight together.  With more
 // rows of A a workgroup takes more weight rows, so that the activations, which every
@@ -213,107 +327,120 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
       }
   }
 
-  if (EPI == EPI_ROPE) {
-    // lane holds row m = 16 mt + r of A and rows 4 g4 + i of each tile: lanes 0-31 the lower
-    // features of the pairs, lanes 32-63 (same m) their partners
-    const int per_head = rope.hd / 16;
-    const int64_t head_step = (int64_t)rope.bs * rope.hd;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      if (MT > 1 && mt != wave) continue;  // another wavefront's column tile
-      const int m = 16 * mt + r;
-      const int mc = m < M ? m : M - 1;
-      const int pos = rope.positions[mc];
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int tile = blockIdx.x * RT + rt;
-        const int head = tile / per_head, j = tile % per_head;
-        const bool rotated = 16 * j < rope.rot && head < rope.nh + rope.nkv;  // values keep the tile layout, unrotated
-        const int f0 = rope_feature(j, 4 * g4, rope.rot);  // first of this lane's 4 consecutive features
-        const int n = head * rope.hd + f0;
-        s16x4 res;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          // the projection is rounded to bfloat16 before the rotation, as where the two are separate kernels
-          const float own = __bfloat162float(__float2bfloat16(
-              acc[rt][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f)));
-          const float other = __shfl_xor(own, 32);  // in every lane
-          float o = own;
-          if (rotated) {
-            const float* angle = rope.cos_sin + ((int64_t)mc * (rope.rot / 2) + 8 * j + (4 * g4 + i) % 8) * 2;
-            const float cs = angle[0], sn = angle[1];
-            o = g4 < 2 ? own * cs - other * sn : own * cs + other * sn;
-          }
-          res[i] = to_bf16_bits(o);
-        }
-        if (m >= M || n >= N) continue;
-        if (head < rope.nh) {
-          *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + n) = res;
-          continue;
-        }
-        const int off = pos % rope.bs;
-        const int64_t page = (int64_t)rope.block_tables[(int64_t)rope.tok_seq[m] * rope.max_blocks + pos / rope.bs] *
-                             rope.nkv * head_step;
-        if (head < rope.nh + rope.nkv) {
-          *reinterpret_cast<s16x4*>(rope.k_cache + page + (head - rope.nh) * head_step + (int64_t)off * rope.hd + f0) = res;
-        } else {
-          short* dst = reinterpret_cast<short*>(rope.v_cache) + page + (head - rope.nh - rope.nkv) * head_step +
-                       (int64_t)f0 * rope.bs + off;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) dst[(int64_t)i * rope.bs] = res[i];
-        }
-      }
-    }
-    return;
-  }
+  skinny_epilogue<MT, RT, EPI>(acc, blockIdx.x * RT, MT > 1 ? wave : -1, out, ldc, bias, b_is_f32, M, N, blockIdx.y,
+                               part_stride, rope);
+}
 
-  const bool vec = ldc % 4 == 0;  // rows of out keep 8- and 16-byte stores aligned
-  // lane holds, per column tile mt, row m = 16 mt + r of A and weight rows 4 g4 + i of each row tile
+// The same product for 17..64 rows of A where there are many weight rows.  With several column
+// tiles the kernel above is held up by the activations, which every workgroup reads again for its
+// few weight rows, and by adding up its four wavefronts' sums.  Here a workgroup takes 128 weight
+// rows, 32 per wavefront over the whole k range, and reads each 128-wide slab of the activations
+// once: all threads load it together and leave it in LDS in the order the matrix instruction
+// wants, where every wavefront reads its fragments with one 16-byte read each (two slabs take
+// turns: the next is fetched while the current one is used).  Weight fragments come straight
+// from memory as above.  Every wavefront ends with whole sums of its own rows.
+template <int MT, int EPI>
+__global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out, int64_t ldc,
+                                                          const bf16_t* __restrict__ A, int64_t lda,
+                                                          const bf16_t* __restrict__ W,
+                                                          const void* __restrict__ bias, int b_is_f32, int M,
+                                                          int N, int K, int k_per_split, int64_t part_stride,
+                                                          SkinnyRope rope) {
+  constexpr int RT = 2, KC = 128;
+  __shared__ bf16x8 a_lds[2][MT][KC / 32][PAE_WAVE];  // [slab][column tile][k step][lane]
+  const int tid = threadIdx.x, lane = tid % PAE_WAVE, wave = tid / PAE_WAVE;
+  const int g4 = lane / 16;
+  const int tile_base = (blockIdx.x * 4 + wave) * RT;  // this wavefront's first tile of 16 weight rows
+  const int k_lo = blockIdx.y * k_per_split;
+  const int k_hi = min(K, k_lo + k_per_split);
+  const int lrow = lane / 4, lkg = lane % 4;
+  const int fetch_from = ((lane % 16) * 4 + lane / 16) * 4;
+  const bf16_t* wrow[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    int n = 16 * (tile_base + rt) + lrow;
+    if (EPI == EPI_ROPE) {
+      const int tile = tile_base + rt, per_head = rope.hd / 16;
+      n = tile / per_head * rope.hd + rope_feature(tile % per_head, lrow, rope.rot);
+    }
+    wrow[rt] = W + (int64_t)(n < N ? n : N - 1) * K;  // rows past N are loaded from the last row and never stored
+  }
+  // the slab of A: thread t brings, per column tile, the 8 elements at k offset 8 (t % 16) of row
+  // t / 16, which lane (t % 16) % 4 * 16 + t / 16 of k step (t % 16) / 4 wants as its B fragment
+  const int arow = tid / 16, achunk = tid % 16;
+  const bf16_t* aptr[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    if (MT > 1 && mt != wave) continue;  // another wavefront's column tile
-    const int m = 16 * mt + r;
-    if (m >= M) continue;
-    if (EPI == EPI_SWIGLU) {
+    const int m = 16 * mt + arow;
+    aptr[mt] = A + (int64_t)(m < M ? m : M - 1) * lda;
+  }
+  const int a_slot = (achunk % 4) * 16 + arow, a_step = achunk / 4;
+
+  f32x4 acc[RT][MT];
 #pragma unroll
-      for (int pair = 0; pair < RT / 2; ++pair) {  // tiles 2 pair (gate) and 2 pair + 1 (up)
-        const int j = (blockIdx.x * (RT / 2) + pair) * 16 + 4 * g4;  // output feature of register 0
-        if (j >= N / 2) continue;                                    // N counts gate and up rows
-        s16x4 v;
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float g = acc[2 * pair][mt][i], u = acc[2 * pair + 1][mt][i];
-          v[i] = to_bf16_bits(g / (1.0f + expf(-g)) * u);
-        }
-        *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j) = v;
-      }
-    } else {
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {};
+  struct Slab {
+    bf16x8 wf[KC / 32][RT], a[MT];
+  };
+  auto load = [&](Slab& b, int kc) {  // loads are unconditional, from clamped addresses
+    const int ka = kc + 8 * achunk;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) b.a[mt] = *reinterpret_cast<const bf16x8*>(aptr[mt] + (ka < K - 8 ? ka : K - 8));
+#pragma unroll
+    for (int st = 0; st < KC / 32; ++st) {
+      const int k = kc + 32 * st + 8 * lkg;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) b.wf[st][rt] = *reinterpret_cast<const bf16x8*>(wrow[rt] + (k < K - 8 ? k : K - 8));
+    }
+  };
+  auto stage = [&](const Slab& b, int buf) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) a_lds[buf][mt][a_step][a_slot] = b.a[mt];
+  };
+  auto multiply = [&](Slab& b, int kc, int buf) {
+#pragma unroll
+    for (int st = 0; st < KC / 32; ++st) {
+      // a lane past the end of the k range zeroes its weight fragment (K and the bounds are multiples of 8)
+      const bool kok = kc + 32 * st + 8 * g4 < k_hi;
+      bf16x8 af[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) af[mt] = a_lds[buf][mt][st][lane];
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
-        const int n = n0 + 16 * rt + 4 * g4;
-        if (n >= N) continue;
-        float v[4];
+        const bf16x8 moved = to_mfma_order(b.wf[st][rt], fetch_from);  // in every lane
+        const bf16x8 w = kok ? moved : zero;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          v[i] = acc[rt][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f);
-        if (EPI == EPI_F32) {
-          float* dst = (float*)out + (int64_t)blockIdx.y * part_stride + (int64_t)m * ldc + n;
-          if (vec && n + 4 <= N) *reinterpret_cast<f32x4*>(dst) = (f32x4){v[0], v[1], v[2], v[3]};
-          else
-            for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = v[i];
-        } else {
-          bf16_t* dst = (bf16_t*)out + (int64_t)m * ldc + n;
-          if (vec && n + 4 <= N) {
-            s16x4 p;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) p[i] = to_bf16_bits(v[i]);
-            *reinterpret_cast<s16x4*>(dst) = p;
-          } else
-            for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = __float2bfloat16(v[i]);
-        }
+        for (int mt = 0; mt < MT; ++mt)
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, af[mt], acc[rt][mt], 0, 0, 0);
       }
     }
+  };
+  // the k range is the same for the whole workgroup: every wavefront passes the same barriers
+  Slab s0, s1;
+  int kc = k_lo;
+  load(s0, kc);
+  stage(s0, 0);
+  __syncthreads();
+  while (true) {
+    const bool more0 = kc + KC < k_hi;
+    if (more0) load(s1, kc + KC);
+    multiply(s0, kc, 0);
+    if (!more0) break;
+    stage(s1, 1);
+    __syncthreads();
+    kc += KC;
+    const bool more1 = kc + KC < k_hi;
+    if (more1) load(s0, kc + KC);
+    multiply(s1, kc, 1);
+    if (!more1) break;
+    stage(s0, 0);
+    __syncthreads();
+    kc += KC;
   }
+  skinny_epilogue<MT, RT, EPI>(acc, tile_base, -1, out, ldc, bias, b_is_f32, M, N, blockIdx.y, part_stride, rope);
 }
 
 // epilogue: 0 bfloat16 out (+bias), 1 float32 out (`splits` partials of `part_stride`
@@ -335,6 +462,31 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + 127) / 128 * 128;
   PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "gemm_skinny: %d k ranges are too many for K=%d", splits, K);
+  // many weight rows and more than 16 rows of A: 128 weight rows a workgroup, activations through LDS
+  // (measured at 1.5B/7B/72B layer sizes: ahead from about one workgroup per compute unit on, behind below)
+  const int medium_groups = (N + 127) / 128;
+  if (mt >= 2 && (int64_t)medium_groups * splits >= 256) {
+    dim3 mgrid(medium_groups, splits);
+#define LAUNCH_MEDIUM(MT, EPI)                                                                                  \
+  gemm_medium_kernel<MT, EPI><<<mgrid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, bias, \
+                                                         b_is_f32, M, N, K, k_per_split, part_stride, rope)
+#define MEDIUM_BY_MT(EPI)                       \
+  switch (mt) {                                 \
+    case 2: LAUNCH_MEDIUM(2, EPI); break;       \
+    case 3: LAUNCH_MEDIUM(3, EPI); break;       \
+    default: LAUNCH_MEDIUM(4, EPI); break;      \
+  }
+    switch (epilogue) {
+      case EPI_BF16: MEDIUM_BY_MT(EPI_BF16); break;
+      case EPI_F32: MEDIUM_BY_MT(EPI_F32); break;
+      case EPI_SWIGLU: MEDIUM_BY_MT(EPI_SWIGLU); break;
+      case EPI_ROPE: MEDIUM_BY_MT(EPI_ROPE); break;
+      default: return pae_fail("gemm_skinny: unknown epilogue %d", epilogue);
+    }
+#undef MEDIUM_BY_MT
+#undef LAUNCH_MEDIUM
+    return pae_check_launch("gemm_medium");
+  }
   dim3 grid((N + 16 * rt - 1) / (16 * rt), splits);
   // four k steps of loads in flight per wavefront: deeper prefetch costs registers and measured slower
 #define LAUNCH(MT, RT, EPI)                                                                                  \
