@@ -154,7 +154,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int hi = min((split + 1) * SPLIT, pos[0] + 1);  // keys [lo, hi), not empty
   const int* table = block_tables + (int64_t)tok_seq[tok] * max_blocks;
   const int g = nh / nkv;
-  const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
+  // (the wavefront's number as a scalar, so that its pages' table entries come by scalar loads)
+  const int lane = threadIdx.x % PAE_WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE);
   const int col = lane % 16, g4 = lane / 16;
 
   bf16x8 qf[1][HD / 32];
@@ -340,7 +341,11 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
   __shared__ float s_acc[3][HD / 16][4][PAE_WAVE];
   __shared__ float s_ml[3][2][PAE_WAVE];
 
-  const int wave = threadIdx.x / PAE_WAVE, lane = threadIdx.x % PAE_WAVE;
+  // the wavefront's number as a scalar: what is computed from it (the keys it takes, their pages'
+  // table entries) then lives in scalar registers and is loaded by scalar loads, which the vector
+  // loads' in-order counter does not wait for (as a vector load, every table lookup waited for all
+  // keys and values in flight)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE), lane = threadIdx.x % PAE_WAVE;
   const int col = lane % 16, g4 = lane / 16;
   const int head = blockIdx.x, kvh = head / (nh / nkv);
   const int seq_row = tiles[blockIdx.y * 3];
@@ -404,14 +409,17 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
     }
   };
   auto load_values = [&](int key0) {
+    const bf16_t* vp[2];
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
       const int key = key0 + 16 * p, kc = key <= hi ? key : key0;
-      const bf16_t* vp = v_cache + page_base(key0, p) + kc % bs;
-#pragma unroll
-      for (int t = 0; t < HD / 16; ++t)
-        reinterpret_cast<bf16x4*>(&vf[t])[p] = *reinterpret_cast<const bf16x4*>(vp + (int64_t)(16 * t + lrow) * bs + 4 * lgrp);
+      vp[p] = v_cache + page_base(key0, p) + kc % bs;
     }
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t)  // in the order of their use
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+        reinterpret_cast<bf16x4*>(&vf[t])[p] = *reinterpret_cast<const bf16x4*>(vp[p] + (int64_t)(16 * t + lrow) * bs + 4 * lgrp);
   };
 
   int key0 = lo + UNIT * wave;  // the same in every lane of a wavefront: the branches on it are uniform
