@@ -498,7 +498,12 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
     for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
       for (int t = 0; t < HD / 16; ++t) asm volatile("" : "+a"(acc[ct][t]));
-    bf16x8 pb[CT];
+    // Column tile by column tile: the weights of one (exponentials, sum, rounding: vector ALU), then
+    // its second product (matrix pipe), so that the next tile's arithmetic can run under this
+    // tile's products.  The values are moved to the instruction's order once, before.
+    bf16x8 va[HD / 16];
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) va[t] = quad_to_mfma_order(vf[t], fetch_from);
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
       float w[8];
@@ -508,15 +513,22 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
         for (int i = 0; i < 4; ++i)
           w[4 * p + i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ct][p][i], scale_log2, -ref[ct]));
       l[ct] += ((w[0] + w[1]) + (w[2] + w[3])) + ((w[4] + w[5]) + (w[6] + w[7]));
-      bf16x2* pairs = reinterpret_cast<bf16x2*>(&pb[ct]);
+      bf16x8 pb;
+      bf16x2* pairs = reinterpret_cast<bf16x2*>(&pb);
 #pragma unroll
       for (int i = 0; i < 4; ++i) pairs[i] = __builtin_convertvector((f32x2){w[2 * i], w[2 * i + 1]}, bf16x2);
+#pragma unroll
+      for (int t = 0; t < HD / 16; ++t) acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[t], pb, acc[ct][t], 0, 0, 0);
     }
+    // Order asked of the compiler's scheduler for the above: the permutes, the first tile's
+    // arithmetic, then one matrix instruction and two vector instructions in turn (left alone it
+    // puts all exponentials first and all products last, and each pipe idles while the other runs).
+    __builtin_amdgcn_sched_group_barrier(0x080, HD / 16 * 4, 0);
+    __builtin_amdgcn_sched_group_barrier(0x002, 20, 0);
 #pragma unroll
-    for (int t = 0; t < HD / 16; ++t) {
-      const bf16x8 va = quad_to_mfma_order(vf[t], fetch_from);
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[ct], acc[ct][t], 0, 0, 0);
+    for (int i = 0; i < CT * (HD / 16); ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
     }
     if (more) load_values(key0 + 4 * UNIT);
   }
