@@ -3,7 +3,7 @@
 The reference has this only in its tests (tests/tiny_model.py:21-50:
 `torch.manual_seed(seed)`, every matrix randn * 0.02, zero biases, unit norm
 weights).  Here biases are drawn as well, so that the bias path carries signal,
-and norm weights may be spread around 1.  Values are drawn in float32 and stored
+and norm weights may be spread about one.  Values are drawn in float32 and stored
 as bfloat16, the precision checkpoints of this family ship in, so that the
 32-bit and the bfloat16 paths start from the same numbers.
 

@@ -169,6 +169,44 @@ from dataclasses import dataclass
 
 
 @dataclass(frozen=True)
+class RoutedSpec(PartSpec):
+    hidden_size: int = 0
+    intermediate_size: int = 0
+    num_experts: int = 2
+    kind: str = "toy_routed"
+
+
+@P.register_feed_forward("toy_routed")
+class RoutedFeedForward(P.Part):
+    """y = down_e(relu(up_e(x))) with e = argmax(router x), router logits in float32: a feed-forward
+    that sends every token to one of several experts.  The products are the framework's own
+    `Linear` (its kernels); the routing is a few library calls (a test part)."""
+
+    def tensors(self, prefix):
+        s = self.spec
+        out = {prefix + "router.weight": (s.num_experts, s.hidden_size)}
+        for e in range(s.num_experts):
+            out[prefix + f"experts.{e}.up.weight"] = (s.intermediate_size, s.hidden_size)
+            out[prefix + f"experts.{e}.down.weight"] = (s.hidden_size, s.intermediate_size)
+        return out
+
+    def bind(self, prefix, weights):
+        from paged_attention_engine_amd.parts.linear import Linear
+        self.router = weights[prefix + "router.weight"].to(device=self.device, dtype=torch.float32)
+        self.up = [Linear(self.matrix(weights[prefix + f"experts.{e}.up.weight"])) for e in range(self.spec.num_experts)]
+        self.down = [Linear(self.matrix(weights[prefix + f"experts.{e}.down.weight"])) for e in range(self.spec.num_experts)]
+
+    def forward(self, ctx, x):
+        choice = (x.float() @ self.router.t()).argmax(-1)  # a function of the token alone
+        out = torch.zeros_like(x)
+        for e in range(self.spec.num_experts):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                out[rows] = self.down[e](torch.relu(self.up[e](x[rows].contiguous())))
+        return out
+
+
+@dataclass(frozen=True)
 class DecaySpec(PartSpec):
     hidden_size: int = 0
     decay: float = 0.5
@@ -243,6 +281,38 @@ def toy_plain_logits(w, c, ids):
         h = plain.rms_norm(x, w[p + "post_attention_layernorm.weight"].double(), c["eps"])
         x = x + plain.swiglu_mlp({k: v.double() for k, v in w.items()}, p, h)
     return plain.linear(plain.rms_norm(x, w["final_norm.weight"].double(), c["eps"]), w["head.weight"].double())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_is_registered_and_built(dtype):
+    """A feed-forward with routing, defined above in this file, goes through the registry and runs
+    on the framework's products; 100 tokens (the many-row path) and 5 (the few-row path)."""
+    torch.manual_seed(11)
+    H, I, E = 64, 96, 3
+    spec = RoutedSpec(hidden_size=H, intermediate_size=I, num_experts=E)
+    part = P.build_part(P.FEED_FORWARDS, "feed-forward", spec, DT[dtype], DEV)
+    names = part.tensors("m.mlp.")
+    assert len(names) == 1 + 2 * E
+    w = {n: (torch.randn(shape) * 0.2).to(DT[dtype]) for n, shape in names.items()}
+    part.bind("m.mlp.", w)
+    router = w["m.mlp.router.weight"].double()
+    for T in (100, 5):
+        x = torch.randn(T, H)
+        # push every token towards one expert, so that no rounding decides the routing
+        target = torch.arange(T) % E
+        x = (x + 3.0 * router[target].float() / router[target].float().norm(dim=1, keepdim=True)).to(DT[dtype])
+        logits = x.double() @ router.t()
+        top2 = logits.topk(2, dim=-1).values
+        assert float((top2[:, 0] - top2[:, 1]).min()) > 0.05
+        choice = logits.argmax(-1)
+        want = torch.zeros(T, H, dtype=torch.float64)
+        for e in range(E):
+            rows = choice == e
+            up, down = w[f"m.mlp.experts.{e}.up.weight"].double(), w[f"m.mlp.experts.{e}.down.weight"].double()
+            want[rows] = torch.relu(x[rows].double() @ up.t()) @ down.t()
+        assert len(set(choice.tolist())) == E
+        got = part.forward(None, x.to(DEV))
+        assert (got.double().cpu() - want).abs().max() <= TOL[dtype] * max(1.0, float(want.abs().max()))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
