@@ -106,13 +106,17 @@ def decode_run(model, cfg, batch: int, ctx: int, steps: int, warmup: int, block_
         result = engine.step()
         assert len(result.decoded) == batch, result
     held_before = sum(engine.cache.num_tokens(s.seq_id) for s in sched.running)
+    generated_before = sum(len(s.generated) for s in sched.running)
     torch.cuda.synchronize()
     start = time.perf_counter()
-    for _ in range(steps):
-        result = engine.step()
+    # the engine's own loop: the next step is decided and launched while the current one runs,
+    # and the clock stops when the last step's tokens are on the host
+    ran = engine.run_steps(steps)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - start
-    assert len(result.decoded) == batch and not result.prefilled and len(sched.running) == batch, result
+    assert ran == steps and len(sched.running) == batch and not any(s.prefilling for s in sched.running)
+    assert sum(len(s.generated) for s in sched.running) - generated_before == batch * steps
+    assert all(t >= 0 for s in sched.running for t in s.generated)
     held_after = sum(engine.cache.num_tokens(s.seq_id) for s in sched.running)
     del engine, sched
     torch.cuda.empty_cache()

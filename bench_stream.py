@@ -69,20 +69,24 @@ def run_stream(model, requests, block_size, num_blocks, max_num_seqs, budget):
     for r in requests:
         if not engine.add_request(r):
             raise SystemExit(f"request {r.request_id} rejected: {engine.events_of(pae.EventKind.REJECT)[-1].detail}")
+    tokens_to_run = sum(r.max_total_len - 1 for r in requests)  # without replays
     torch.cuda.synchronize()
     start = time.perf_counter()
-    steps = tokens_run = 0
+    steps = 0
     last = start
-    while engine.scheduler.waiting or engine.scheduler.running:
-        result = engine.step()
-        steps += 1
-        tokens_run += result.batched_token_cost
+    sched = engine.scheduler
+    while sched.waiting or sched.running:
+        # the engine's own loop (the next step is launched while the current one runs), in
+        # stretches so that a long run reports where it is
+        steps += engine.run_steps(64)
         if time.perf_counter() - last > 30:
             last = time.perf_counter()
-            print(f"[stream] step {steps}: {len(engine.finished)} finished, {result.running} running, "
-                  f"{result.waiting} waiting, {result.free_blocks} free pages", file=sys.stderr, flush=True)
+            print(f"[stream] step {steps}: {len(engine.finished)} finished, {len(sched.running)} running, "
+                  f"{len(sched.waiting)} waiting, {engine.cache.min_free_blocks()} free pages",
+                  file=sys.stderr, flush=True)
     torch.cuda.synchronize()
     wall = time.perf_counter() - start
+    tokens_run = tokens_to_run + sum(int(e.detail.split()[1]) for e in engine.events_of(pae.EventKind.RECOMPUTE))
     outputs = {rid: tuple(seq.generated) for rid, seq in engine.finished.items()}
     stats = dict(wall_s=wall, steps=steps, mean_batch_tokens=tokens_run / max(steps, 1),
                  preemptions=len(engine.events_of(pae.EventKind.PREEMPT)),

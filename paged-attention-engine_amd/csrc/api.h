@@ -15,6 +15,7 @@ int pae_add_rmsnorm(int dtype, void* residual, const void* delta, int parts, int
                     const void* weight, int w_is_f32, float eps, const int* rows, void* out, int num_rows,
                     int hidden, int write_residual, hipStream_t stream);
 int pae_residual_add(int dtype, void* residual, const void* delta, int64_t n, hipStream_t stream);
+int pae_scatter_i32(int* dst, const int* dst_idx, const int* src, const int* src_idx, int n, hipStream_t stream);
 int pae_rope_table(float* cos_sin, const int* positions, const float* inv_freq, int num_tokens, int half,
                    hipStream_t stream);
 int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int rot,

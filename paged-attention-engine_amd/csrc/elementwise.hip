@@ -222,6 +222,23 @@ extern "C" int pae_residual_add(int dtype, void* residual, const void* delta, in
   return pae_check_launch("residual_add");
 }
 
+// ---------------------------------------------------------------- token ids that are still on the device
+// dst[dst_idx[i]] = src[src_idx[i]]: a step whose input token was sampled by the step before takes
+// it from that step's output without a round trip through the host.
+__global__ void scatter_i32_kernel(int* __restrict__ dst, const int* __restrict__ dst_idx,
+                                   const int* __restrict__ src, const int* __restrict__ src_idx, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[dst_idx[i]] = src[src_idx[i]];
+}
+
+extern "C" int pae_scatter_i32(int* dst, const int* dst_idx, const int* src, const int* src_idx, int n,
+                               hipStream_t stream) {
+  PAE_REQUIRE(n >= 0, "scatter_i32: n=%d", n);
+  if (n == 0) return 0;
+  scatter_i32_kernel<<<(n + 255) / 256, 256, 0, stream>>>(dst, dst_idx, src, src_idx, n);
+  return pae_check_launch("scatter_i32");
+}
+
 // ---------------------------------------------------------------- rotation + cache write
 // qkv row t holds [q heads | k heads | v heads], each head `hd` wide.  Query and
 // key heads are rotated over their first `rot` features in pairs (i, i + rot/2):

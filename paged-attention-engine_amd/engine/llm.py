@@ -64,8 +64,24 @@ class Engine:
     def step(self) -> StepResult:
         return self.scheduler.step()
 
-    def run_to_completion(self, max_steps: int = 100_000) -> Dict[str, Tuple[int, ...]]:
+    def run_to_completion(self, max_steps: int = 100_000, overlap: bool = True) -> Dict[str, Tuple[int, ...]]:
+        """Run until every request has finished.  With `overlap` (and no stop tokens, no recorded
+        logits) the next step is decided and launched while the current one runs; decisions and
+        tokens are those of stepping one by one."""
+        if overlap and self.scheduler.can_overlap():
+            self.scheduler.run_overlapped(max_steps)
+            return {rid: tuple(seq.generated) for rid, seq in self.scheduler.finished.items()}
         return self.scheduler.run_to_completion(max_steps)
+
+    def run_steps(self, count: int, overlap: bool = True) -> int:
+        """At most `count` steps (fewer if nothing is left); returns how many ran."""
+        if overlap and self.scheduler.can_overlap():
+            return self.scheduler.run_overlapped(count, until_idle=False)
+        done = 0
+        while done < count and (self.scheduler.waiting or self.scheduler.running):
+            self.scheduler.step()
+            done += 1
+        return done
 
     def events_of(self, kind: EventKind):
         return self.scheduler.events_of(kind)

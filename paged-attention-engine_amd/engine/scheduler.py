@@ -42,6 +42,10 @@ from ..cache.manager import CacheManager
 from ..config.engine_config import ADMISSION_MARGIN_BLOCKS
 
 
+# A generated token whose value is still on the device (see `Scheduler.run_overlapped`).
+PENDING = -1
+
+
 class EventKind(Enum):
     ADMIT = "admit"
     FINISH = "finish"
@@ -330,14 +334,15 @@ class Scheduler:
         self._log(EventKind.FINISH, seq, f"{len(seq.generated)} tokens, freed {freed} blocks")
 
     # ------------------------------------------------------------------ the step
-    def step(self) -> StepResult:
+    def _plan_batch(self):
+        """Decide a step: what runs, who is evicted, who is admitted.  Pages are reserved and
+        the work is queued; nothing has run yet."""
         self._step += 1
         self._pending = []
         self._pending_tokens = 0
         preempted: List[str] = []
         deferred: List[str] = []
         admitted: List[Sequence] = []
-        finished_before = set(self.finished)
 
         # 1. sequences already running, in running order: decodes and prompt portions
         for want_prefill in (False, True):
@@ -375,32 +380,32 @@ class Scheduler:
             admitted.append(head)
             self._plan(head, min(head.history_len, budget))
 
-        # 3. one pass of the model for everything planned
         batch = self._pending
         self._pending = []
         tokens_run, self._pending_tokens = self._pending_tokens, 0
-        if batch:
-            results = self.executor.execute(batch, self.record_logits)
-            if len(results) != len(batch):
-                raise AssertionError(f"executor returned {len(results)} results for {len(batch)} items")
-            for work, result in zip(batch, results):
-                seq = work.seq
-                seq.num_computed += len(work.token_ids)
-                self.cache.release_passed(seq.seq_id)
-                if not work.samples:
-                    continue
-                token, row = result if isinstance(result, tuple) else (result, None)
-                if token is None:
-                    raise AssertionError(f"{seq.request_id}: executor returned no token for a sampling item")
-                seq.prefilling = False
-                if self.record_logits:
-                    seq.step_logits.append(row)
-                seq.generated.append(int(token))
-                if int(token) in seq.request.stop_token_ids:
-                    seq.stopped = True
-                if seq.is_finished:
-                    self._finish(seq)
+        return batch, tokens_run, preempted, deferred, admitted
 
+    def _advance(self, work: ScheduledWork, token: Optional[int], row=None) -> None:
+        """What a work item that has run (or is sure to) changes: the sequence's progress, the
+        pages a window has passed, and for an item that samples its new token (PENDING while
+        the value is still on the device), a stop, the end."""
+        seq = work.seq
+        seq.num_computed += len(work.token_ids)
+        self.cache.release_passed(seq.seq_id)
+        if not work.samples:
+            return
+        if token is None:
+            raise AssertionError(f"{seq.request_id}: executor returned no token for a sampling item")
+        seq.prefilling = False
+        if self.record_logits:
+            seq.step_logits.append(row)
+        seq.generated.append(int(token))
+        if int(token) in seq.request.stop_token_ids:
+            seq.stopped = True
+        if seq.is_finished:
+            self._finish(seq)
+
+    def _result(self, batch, tokens_run, preempted, deferred, admitted, finished_before) -> StepResult:
         return StepResult(
             step=self._step,
             admitted=tuple(s.request_id for s in admitted),
@@ -415,6 +420,71 @@ class Scheduler:
             batched_token_cost=tokens_run,
             prefilled=tuple(w.seq.request_id for w in batch if w.is_prefill),
         )
+
+    def step(self) -> StepResult:
+        finished_before = set(self.finished)
+        batch, tokens_run, preempted, deferred, admitted = self._plan_batch()
+        # one pass of the model for everything planned
+        if batch:
+            results = self.executor.execute(batch, self.record_logits)
+            if len(results) != len(batch):
+                raise AssertionError(f"executor returned {len(results)} results for {len(batch)} items")
+            for work, result in zip(batch, results):
+                token, row = result if isinstance(result, tuple) else (result, None)
+                self._advance(work, token if work.samples else None, row)
+        return self._result(batch, tokens_run, preempted, deferred, admitted, finished_before)
+
+    # ------------------------------------------------------------------ steps that overlap
+    def can_overlap(self) -> bool:
+        """Whether `run_overlapped` may be used: the executor can launch without waiting, no
+        logits are recorded, and no request stops on a token's value."""
+        every = list(self.waiting) + list(self.running)
+        return (hasattr(self.executor, "launch") and not self.record_logits
+                and not any(s.request.stop_token_ids for s in every))
+
+    def run_overlapped(self, max_steps: int = 100_000, until_idle: bool = True) -> int:
+        """Steps of which the next is decided and launched while the current one runs.
+
+        What a step decides depends on the step before only through counts (who has how many
+        tokens, who ends at `max_new_tokens`, which pages are free), never through a token's
+        value, as long as no request has stop tokens: so after a step is launched its sequences
+        are advanced with PENDING in place of their new tokens, the next step is planned and
+        launched (the device hands the sampled ids over: `executor.launch`), and only then the
+        host waits for the earlier step's tokens and writes them over the PENDINGs.  Decisions,
+        events and tokens are those of `step()` called in a loop; the GPU does not wait for
+        the host between steps.  Runs until nothing is left (or `max_steps` steps, with
+        `until_idle=False`); returns the number of steps."""
+        if not self.can_overlap():
+            raise RuntimeError("run_overlapped needs an executor with launch(), no recorded logits and no stop tokens")
+        steps = 0
+        in_flight = None  # (launched step, its sampling work items)
+        while (self.waiting or self.running) and steps < max_steps:
+            batch, _, _, _, _ = self._plan_batch()
+            steps += 1
+            launched = self.executor.launch(batch, in_flight) if batch else None
+            for work in batch:
+                self._advance(work, PENDING if work.samples else None)
+            if in_flight is not None:
+                self._settle(in_flight)
+            in_flight = launched
+            if not batch and in_flight is None and until_idle:
+                raise RuntimeError(f"no progress: {len(self.waiting)} waiting, {len(self.running)} running")
+        if in_flight is not None:
+            self._settle(in_flight)
+        if until_idle and (self.waiting or self.running):
+            raise RuntimeError(f"no progress after {max_steps} steps: {len(self.waiting)} waiting, "
+                               f"{len(self.running)} running")
+        return steps
+
+    def _settle(self, launched) -> None:
+        """The tokens of a launched step have arrived: write them where PENDING stands."""
+        tokens = launched.wait()
+        for work, token in zip(launched.sampling, tokens):
+            seq = work.seq
+            at = work.positions[-1] + 1 - seq.request.prompt_len  # index of this item's token among the generated
+            if seq.generated[at] != PENDING:
+                raise AssertionError(f"{seq.request_id}: token {at} was settled twice")
+            seq.generated[at] = int(token)
 
     def run_to_completion(self, max_steps: int = 100_000) -> Dict[str, Tuple[int, ...]]:
         steps = 0

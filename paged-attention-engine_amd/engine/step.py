@@ -25,6 +25,7 @@ from ..parts import StepContext
 from .model import Model
 
 
+from ..kernels import lib as K
 from ..kernels.lib import PREFILL_TILE  # tokens per run of the prefill attention kernel
 
 
@@ -63,12 +64,18 @@ class StepRunner:
         self._graphs: Dict[tuple, _CapturedStep] = {}
         self.graph_replays = 0
 
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry],
+            feeds: Optional[Tuple[torch.Tensor, Sequence[Tuple[int, int]]]] = None) -> torch.Tensor:
         """Run one step.  Every entry's tokens must already be reserved in the
         cache (`cache.reserve(seq_id, len(token_ids))`), and they are the last
         tokens reserved.  Returns float32 logits [number of wanted places, vocab]
         in the order of the entries and of each entry's `want`.  The tensor may be
-        overwritten by the next call."""
+        overwritten by the next call.
+
+        `feeds = (tokens, [(place, row), ...])`: token ids that are still on the device
+        (an int32 tensor, the step before's samples): the flat token at `place` (counting
+        through the entries) is `tokens[row]`, whatever the entry says there; at most one
+        per sequence.  Nothing waits for the host to see those ids."""
         cache = self.cache
         ids: List[int] = []
         positions: List[int] = []
@@ -125,7 +132,13 @@ class StepRunner:
             tables.append((width, per_seq))
 
         # one staging buffer, one copy to the device
-        flat: List[int] = ids + positions + tok_seq + slots + rows + decode_tokens + tiles
+        # places and rows of token ids that come from the device, padded to one per sequence
+        fed = list(feeds[1]) if feeds is not None else []
+        if len(fed) > S or any(not (0 <= place < T and 0 <= row < feeds[0].numel()) for place, row in fed):
+            raise ValueError("feeds: at most one per sequence, places within the step, rows within the tokens")
+        fed_places = [place for place, _ in fed] + [0] * (S - len(fed))
+        fed_rows = [row for _, row in fed] + [0] * (S - len(fed))
+        flat: List[int] = ids + positions + tok_seq + slots + rows + decode_tokens + tiles + fed_places + fed_rows
         for width, per_seq in tables:
             for table in per_seq:
                 flat.extend(table)
@@ -155,6 +168,9 @@ class StepRunner:
 
         d_ids, d_pos, d_seq, d_slots, d_rows = take(T), take(T), take(T), take(S), take(len(rows))
         d_decode, d_tiles = take(len(decode_tokens)), take(len(tiles)).view(-1, 3)
+        d_fed_places, d_fed_rows = take(S), take(S)
+        if fed:
+            K.scatter_int32(d_ids, d_fed_places, feeds[0], d_fed_rows, len(fed))
         block_tables: Dict[int, torch.Tensor] = {}
         for group, (width, _) in zip(cache.groups, tables):
             block_tables[group.index] = take(S * width).view(S, width)

@@ -54,6 +54,7 @@ def _declare(lib) -> None:
         "pae_embedding": [I, P, P, P, I, I, I, P],
         "pae_add_rmsnorm": [I, P, P, I, L, P, I, F, P, P, I, I, I, P],
         "pae_residual_add": [I, P, P, L, P],
+        "pae_scatter_i32": [P, P, P, P, I, P],
         "pae_rope_table": [P, P, P, I, I, P],
         "pae_rope_kv_write": [I, P, L, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P],
         "pae_swiglu": [I, P, P, I, I, I, P],
@@ -169,6 +170,17 @@ def residual_add(residual: torch.Tensor, delta: torch.Tensor) -> None:
     assert residual.is_contiguous() and delta.is_contiguous()
     _check(library().pae_residual_add(code_of(delta.dtype), residual.data_ptr(), delta.data_ptr(),
                                       residual.numel(), _stream()))
+
+
+def scatter_int32(dst: torch.Tensor, dst_idx: torch.Tensor, src: torch.Tensor, src_idx: torch.Tensor, n: int) -> None:
+    """dst[dst_idx[i]] = src[src_idx[i]] for i < n (int32 everywhere; the index lists may be longer than n).
+    The caller vouches for the indices: they are not checked on the device."""
+    _gpu(dst, dst_idx, src, src_idx)
+    for t in (dst, dst_idx, src, src_idx):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert 0 <= n <= min(dst_idx.numel(), src_idx.numel())
+    _check(library().pae_scatter_i32(dst.data_ptr(), dst_idx.data_ptr(), src.data_ptr(), src_idx.data_ptr(), n,
+                                     _stream()))
 
 
 def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:

@@ -35,9 +35,39 @@ def uniform_for(seed: int, request_id: str, index: int) -> float:
     return (_splitmix64(key ^ (index & _MASK)) >> 40) / float(1 << 24)
 
 
+class SampledTokens:
+    """A step's tokens, sampled on the device and on their way to the host."""
+
+    def __init__(self, on_device: torch.Tensor) -> None:
+        self.on_device = on_device  # int32 [R]; what the next step may be fed from
+        self._host = torch.empty(on_device.shape, dtype=torch.int32, pin_memory=True)
+        self._host.copy_(on_device, non_blocking=True)
+        self._arrived = torch.cuda.Event()
+        self._arrived.record()
+
+    def wait(self) -> list:
+        self._arrived.synchronize()
+        return self._host.tolist()
+
+
 class Sampler:
     def __init__(self, device) -> None:
         self.device = device
+
+    def sample_on_device(self, logits: torch.Tensor, temperatures: Sequence[float],
+                         uniforms: Sequence[float]) -> SampledTokens:
+        """As `sample`, without waiting: the tokens stay on the device for the next step and
+        come to the host behind an event."""
+        rows = logits.shape[0]
+        tokens = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        if rows:
+            if any(t > 0 for t in temperatures):
+                params = torch.tensor([list(temperatures), list(uniforms)], dtype=torch.float32).to(
+                    logits.device, non_blocking=True)
+                K.sample(tokens, logits, params[0], params[1])
+            else:
+                K.sample(tokens, logits, None, None)
+        return SampledTokens(tokens)
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float],
                uniforms: Sequence[float]) -> list:

@@ -198,6 +198,41 @@ def test_preemption_with_recompute_is_transparent(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,num_blocks", [("B", 60), ("B", 14), ("C", 40)])
+def test_overlapped_steps_give_the_tokens_of_single_steps(tmp_path, name, num_blocks, dtype):
+    """`run_to_completion` launches the next step before it has seen the current one's tokens
+    (the sampled ids go from step to step on the device).  Greedy and temperature requests,
+    prompts cut into portions, a pool so small that requests are evicted and replayed: tokens
+    and events are those of `step()` in a loop, bit for bit, because the same kernels run on
+    the same inputs."""
+    folder = helpers.make_model_folder(tmp_path, name)
+    cfg = helpers.TINY[name][0]
+    model = pae.load_model(folder, dtype)
+    shapes = [(3, 12, 0.0), (9, 30, 0.8), (40, 20, 0.0), (64, 17, 0.7), (2, 40, 0.0), (27, 25, 1.1), (50, 33, 0.0)]
+    requests = [pae.Request(f"r{i}", tuple(tokens_of(cfg, n, 70 + i)), new, temp, seed=i)
+                for i, (n, new, temp) in enumerate(shapes)]
+
+    def run(overlap):
+        engine = pae.Engine(model, dtype=dtype, block_size=8, num_blocks=num_blocks, max_num_seqs=4,
+                            max_num_batched_tokens=32)
+        for r in requests:
+            assert engine.add_request(r)
+        assert engine.scheduler.can_overlap()
+        out = engine.run_to_completion(overlap=overlap)
+        events = [(e.step, e.kind, e.request_id, e.detail) for e in engine.scheduler.events]
+        assert all(n == num_blocks for n in engine.cache.free_blocks())  # every group's pool is whole again
+        return out, events, engine.executor.runner.graph_replays
+
+    single, overlapped = run(False), run(True)
+    assert single[0] == overlapped[0] and single[1] == overlapped[1]
+    assert all(len(single[0][r.request_id]) == r.max_new_tokens for r in requests)
+    assert all(0 <= t < cfg["vocab_size"] for tokens in overlapped[0].values() for t in tokens)
+    if num_blocks == 14:
+        assert any(kind is pae.EventKind.PREEMPT for _, kind, _, _ in single[1])
+    assert overlapped[2] > 0  # decode steps were replayed graphs fed from the device
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "D"])
 def test_replayed_graphs_equal_eager_steps(tmp_path, name, dtype):
     """Decode steps replayed as HIP graphs, with eager work and synchronisation between the

@@ -299,3 +299,100 @@ def test_temperature_draws_depend_on_seed_request_and_index_only():
     assert all(0.0 <= u < 1.0 for u in a) and 0.35 < sum(a) / len(a) < 0.65
     assert a != [uniform_for(6, "r1", i) for i in range(200)]
     assert a != [uniform_for(5, "r2", i) for i in range(200)]
+
+
+# ------------------------------------------------------------------ steps that overlap
+class LaunchingExecutor(StubExecutor):
+    """The stub with the asynchronous half of the executor's surface: `launch` returns at once,
+    a token id that reads PENDING is resolved from the step before (as the device does it), and
+    the tokens are only handed out by `wait`."""
+
+    class Launched:
+        def __init__(self, tokens, sampling):
+            self._tokens, self.sampling = tokens, sampling
+            self.row_of = {id(w.seq): k for k, w in enumerate(sampling)}
+            self.waited = False
+
+        def wait(self):
+            self.waited = True
+            return list(self._tokens)
+
+    def launch(self, work, previous=None):
+        from paged_attention_engine_amd.engine.scheduler import PENDING
+        self.calls += 1
+        self.batches.append([(w.seq.request_id, len(w.token_ids), w.positions[0]) for w in work])
+        assert previous is None or not previous.waited, "the step before must still be in flight when the next is launched"
+        tokens, sampling = [], []
+        for w in work:
+            held = self.cache.num_tokens(w.seq.seq_id)
+            assert w.positions == tuple(range(held - len(w.token_ids), held))
+            ids = list(w.token_ids)
+            for i, t in enumerate(ids):
+                if t == PENDING:
+                    ids[i] = previous._tokens[previous.row_of[id(w.seq)]]
+            assert all(0 <= t < VOCAB for t in ids)
+            if w.samples:
+                tokens.append((ids[-1] * 7 + w.positions[-1] * 13 + 1) % VOCAB)
+                sampling.append(w)
+        return self.Launched(tokens, sampling)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_overlapped_steps_decide_and_generate_what_single_steps_do(seed):
+    """Random streams in pools from ample to tight (preemption, replay in portions, deferral):
+    the loop that launches the next step before it has seen the current one's tokens makes the
+    same batches, logs the same events and ends with the same tokens as `step()` in a loop."""
+    import random
+    rng = random.Random(seed)
+    reqs = [request(f"r{i}", rng.randint(1, 30), rng.randint(1, 25)) for i in range(rng.randint(3, 9))]
+    num_blocks = rng.choice([16, 24, 40, 200])
+    kw = dict(max_num_seqs=rng.choice([None, 2, 4]), max_num_batched_tokens=rng.choice([None, 7, 16]))
+
+    def run(overlapped):
+        cache = CacheManager([PagedSpec(1, 1, None)], [None], 4, num_blocks, 64, device=None)
+        executor = LaunchingExecutor(cache)
+        sched = Scheduler(executor, cache, **kw)
+        for r in reqs:
+            sched.add_request(r)
+        if overlapped:
+            assert sched.can_overlap()
+            steps = sched.run_overlapped()
+        else:
+            steps = 0
+            while sched.waiting or sched.running:
+                sched.step()
+                steps += 1
+        tokens = {rid: tuple(s.generated) for rid, s in sched.finished.items()}
+        events = [(e.step, e.kind, e.request_id, e.detail, e.free_blocks, e.running, e.waiting) for e in sched.events]
+        assert tuple(cache.free_blocks()) == (num_blocks,)
+        return steps, tokens, events, executor.batches
+
+    one, two = run(False), run(True)
+    assert one[0] == two[0] and one[1] == two[1] and one[3] == two[3]
+    assert one[2] == two[2]
+    for r in reqs:
+        if r.request_id in one[1]:
+            assert one[1][r.request_id] == expected_tokens(r)
+
+
+def test_overlapped_steps_need_requests_without_stop_tokens():
+    sched, _, _ = make(40)
+    sched.executor = LaunchingExecutor(sched.cache)
+    sched.add_request(request("a", 3, 4, stop_token_ids=(5,)))
+    assert not sched.can_overlap()
+    with pytest.raises(RuntimeError):
+        sched.run_overlapped()
+    plain, _, _ = make(40)  # the stub without launch()
+    plain.add_request(request("a", 3, 4))
+    assert not plain.can_overlap()
+
+
+def test_overlapped_steps_stop_after_a_given_number():
+    sched, _, _ = make(40)
+    sched.executor = LaunchingExecutor(sched.cache)
+    sched.add_request(request("a", 3, 10))
+    assert sched.run_overlapped(4, until_idle=False) == 4
+    seq = sched.running[0]
+    assert len(seq.generated) == 4 and all(t >= 0 for t in seq.generated)  # every token has been settled
+    assert sched.run_overlapped(100, until_idle=False) == 6 and "a" in sched.finished
+    assert tuple(sched.finished["a"].generated) == expected_tokens(request("a", 3, 10))
