@@ -4,17 +4,20 @@
 // Both kernels work on transposed tiles so that the softmax output can feed the
 // second product without leaving registers:
 //   S^T[16 keys x 16 columns] = K[16 keys x hd] * Q^T        (MFMA 16x16x32, k = hd)
-//   O^T[hd x 16 columns]     += V^T[hd x 16 keys] * P^T       (MFMA 16x16x16, k = keys)
+//   O^T[hd x 16 columns]     += V^T[hd x keys] * P^T          (k = 16 keys in the decode kernel,
+//                                                             32 keys of two pages in the prefill kernel)
 // The accumulator layout of S^T (lane = column, registers = 4 consecutive keys) is
 // exactly the B-operand layout of the second product.  A "column" is one (token,
 // query head); the 16 keys of a tile are one cache page (or a 16-key slice of a
 // larger page).  Keys live as [block][kv head][page][hd], values transposed as
-// [block][kv head][hd][page], so both A operands are contiguous per lane.
+// [block][kv head][hd][page], so both A operands are contiguous in memory; they are loaded
+// with a quad of lanes on contiguous bytes and moved to the instruction's lane order by
+// cross-lane permutes (see `load_kv_tile`).
 //
 // decode:  one workgroup per (sequence with a single new token, kv head, split of
 //          the keys); the columns are the query heads that share the kv head, so a
 //          page is read once for all of them.  Four wavefronts take pages in turn
-//          and merge in LDS; the last workgroup to finish merges the splits.  Splits
+//          and merge in LDS; a second small kernel merges the splits.  Splits
 //          start at multiples of the split length from position 0.
 // prefill: one workgroup per (up to 64 consecutive tokens of a sequence, query head), whose
 //          wavefronts share out the keys (see there).

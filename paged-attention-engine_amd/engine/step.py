@@ -14,19 +14,16 @@ reserved room for every token (:414-417), so positions are the run
 from __future__ import annotations
 
 from array import array
-
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
 from ..cache.manager import CacheManager
-from ..parts import StepContext
-from .model import Model
-
-
 from ..kernels import lib as K
 from ..kernels.lib import PREFILL_TILE  # tokens per run of the prefill attention kernel
+from ..parts import StepContext
+from .model import Model
 
 
 @dataclass(frozen=True)
