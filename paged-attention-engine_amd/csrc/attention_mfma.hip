@@ -91,10 +91,12 @@ __device__ __forceinline__ void attn_tile(AttnState<HD, CT>& st, const bf16x8 (&
   }
 }
 
-// Loads are made with the lane order (row = lane / 4, group = lane % 4), so that the four lanes of
-// a quad read contiguous bytes (64 of a key row, 32 of a value row) and the memory pipeline sees
-// one access for them; `kv_to_mfma_order` then moves every register to the order the matrix
-// instruction wants (row = lane % 16, group = lane / 16) with one cross-lane permute each.
+// Keys are loaded with the lane order (row = lane / 4, group = lane % 4), so that the four lanes of
+// a quad read 64 contiguous bytes of a key row and the memory pipeline sees one access for them;
+// `keys_to_mfma_order` then moves every register to the order the matrix instruction wants
+// (row = lane % 16, group = lane / 16) with one cross-lane permute each.  Values are loaded in the
+// instruction's order at once: a quad's four 8-byte pieces lie in rows 2 * page size bytes apart,
+// one 128-byte line at page size 16, which costs the pipeline no more and saves the permutes.
 template <int HD>
 __device__ __forceinline__ void load_kv_tile(bf16x8 (&kf)[HD / 32], s16x4 (&vf)[HD / 16], const bf16_t* kp,
                                              const bf16_t* vp, int vstride) {
@@ -104,13 +106,12 @@ __device__ __forceinline__ void load_kv_tile(bf16x8 (&kf)[HD / 32], s16x4 (&vf)[
   for (int j = 0; j < HD / 32; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(kp + r * HD + 32 * j + 8 * g);
 #pragma unroll
   for (int t = 0; t < HD / 16; ++t)
-    vf[t] = *reinterpret_cast<const s16x4*>(vp + (int64_t)(16 * t + r) * vstride + 4 * g);
+    vf[t] = *reinterpret_cast<const s16x4*>(vp + (int64_t)(16 * t + lane % 16) * vstride + 4 * (lane / 16));
 }
 
 template <int HD>
-__device__ __forceinline__ void kv_to_mfma_order(bf16x8 (&kf)[HD / 32], s16x4 (&vf)[HD / 16]) {
+__device__ __forceinline__ void keys_to_mfma_order(bf16x8 (&kf)[HD / 32]) {
   typedef __attribute__((ext_vector_type(4))) int i32x4;
-  typedef __attribute__((ext_vector_type(2))) int i32x2;
   const int lane = threadIdx.x % PAE_WAVE;
   const int fetch_from = ((lane % 16) * 4 + lane / 16) * 4;  // byte address of the source lane
 #pragma unroll
@@ -119,13 +120,6 @@ __device__ __forceinline__ void kv_to_mfma_order(bf16x8 (&kf)[HD / 32], s16x4 (&
 #pragma unroll
     for (int i = 0; i < 4; ++i) raw[i] = __builtin_amdgcn_ds_bpermute(fetch_from, raw[i]);
     kf[j] = *reinterpret_cast<bf16x8*>(&raw);
-  }
-#pragma unroll
-  for (int t = 0; t < HD / 16; ++t) {
-    i32x2 raw = *reinterpret_cast<i32x2*>(&vf[t]);
-#pragma unroll
-    for (int i = 0; i < 2; ++i) raw[i] = __builtin_amdgcn_ds_bpermute(fetch_from, raw[i]);
-    vf[t] = *reinterpret_cast<s16x4*>(&raw);
   }
 }
 
@@ -192,7 +186,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
   for (int j = 0; j < TPW; ++j) {
     const int tile = tile_lo + wave + 4 * j;
-    kv_to_mfma_order<HD>(kf[j], vf[j]);  // in every lane of the wavefront, used or not
+    keys_to_mfma_order<HD>(kf[j]);  // in every lane of the wavefront, used or not
     if (tile < tile_hi) attn_tile<HD, 1>(st, kf[j], vf[j], qf, tile * 16, pos, start, scale_log2);
   }
 
@@ -388,10 +382,14 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
     for (int t = 0; t < HD / 16; ++t) acc[ct][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
 
-  // Loads in the order (row = lane / 4, group = lane % 4): a quad reads 64 contiguous bytes of a
-  // key row, or 32 of a value row.  kf[p][j]: keys of page p, features 32 j ..; vf[t]: features
-  // 16 t .., whose 8 k slots per lane are keys 4 g4 .. + 3 of the first page followed by the same
-  // four of the second, exactly the scores a lane holds after the first product.
+  // Keys are loaded in the order (row = lane / 4, group = lane % 4), in which a quad of lanes reads
+  // 64 contiguous bytes of a key row, and moved to the instruction's order by a permute.  kf[p][j]:
+  // keys of page p, features 32 j ..  Values are loaded in the instruction's own order, feature
+  // 16 t + lane % 16, keys 4 (lane / 16) .. + 3 of both pages: a quad's four pieces then lie in one
+  // 128-byte line (value rows are 2 * page size bytes apart), which the memory pipeline takes as
+  // well as contiguous ones, and the permutes are saved (378 -> 353 us at 8,192 tokens; keys, whose
+  // rows are 2 * head_dim bytes apart, gain nothing without theirs).  vf[t]'s 8 k slots per lane
+  // are exactly the scores the lane holds after the first product.
   const int lrow = lane / 4, lgrp = lane % 4;
   const int fetch_from = ((lane % 16) * 4 + lane / 16) * 4;
   const int page_elems = bs * HD;
@@ -422,7 +420,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
     for (int t = 0; t < HD / 16; ++t)  // in the order of their use
 #pragma unroll
       for (int p = 0; p < 2; ++p)
-        reinterpret_cast<bf16x4*>(&vf[t])[p] = *reinterpret_cast<const bf16x4*>(vp[p] + (int64_t)(16 * t + lrow) * bs + 4 * lgrp);
+        reinterpret_cast<bf16x4*>(&vf[t])[p] = *reinterpret_cast<const bf16x4*>(vp[p] + (int64_t)(16 * t + col) * bs + 4 * g4);
   };
 
   int key0 = lo + UNIT * wave;  // the same in every lane of a wavefront: the branches on it are uniform
@@ -503,10 +501,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
       for (int t = 0; t < HD / 16; ++t) asm volatile("" : "+a"(acc[ct][t]));
     // Column tile by column tile: the weights of one (exponentials, sum, rounding: vector ALU), then
     // its second product (matrix pipe), so that the next tile's arithmetic can run under this
-    // tile's products.  The values are moved to the instruction's order once, before.
-    bf16x8 va[HD / 16];
-#pragma unroll
-    for (int t = 0; t < HD / 16; ++t) va[t] = quad_to_mfma_order(vf[t], fetch_from);
+    // tile's products.
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
       float w[8];
@@ -521,12 +516,11 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) pairs[i] = __builtin_convertvector((f32x2){w[2 * i], w[2 * i + 1]}, bf16x2);
 #pragma unroll
-      for (int t = 0; t < HD / 16; ++t) acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[t], pb, acc[ct][t], 0, 0, 0);
+      for (int t = 0; t < HD / 16; ++t) acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t], pb, acc[ct][t], 0, 0, 0);
     }
-    // Order asked of the compiler's scheduler for the above: the permutes, the first tile's
-    // arithmetic, then one matrix instruction and two vector instructions in turn (left alone it
-    // puts all exponentials first and all products last, and each pipe idles while the other runs).
-    __builtin_amdgcn_sched_group_barrier(0x080, HD / 16 * 4, 0);
+    // Order asked of the compiler's scheduler for the above: the first tile's arithmetic, then one
+    // matrix instruction and two vector instructions in turn (left alone it puts all exponentials
+    // first and all products last, and each pipe idles while the other runs).
     __builtin_amdgcn_sched_group_barrier(0x002, 20, 0);
 #pragma unroll
     for (int i = 0; i < CT * (HD / 16); ++i) {
