@@ -33,13 +33,19 @@ class ModelExecutor:
         self.runner = StepRunner(model, cache)
         self.sampler = Sampler(model.device)
 
+    @staticmethod
+    def _uniforms(sampling: Sequence) -> List[float]:
+        """The draw of every item that samples with a temperature (greedy items need none)."""
+        return [uniform_for(w.seq.request.seed, w.seq.request_id, len(w.seq.generated))
+                if w.seq.request.temperature > 0 else 0.0 for w in sampling]
+
     def execute(self, work: Sequence, record_logits: bool = False) -> List:
         entries = [StepEntry(w.seq.seq_id, w.token_ids, (len(w.token_ids) - 1,) if w.samples else ())
                    for w in work]
         logits = self.runner.run(entries)
         sampling = [w for w in work if w.samples]
         temperatures = [w.seq.request.temperature for w in sampling]
-        uniforms = [uniform_for(w.seq.request.seed, w.seq.request_id, len(w.seq.generated)) for w in sampling]
+        uniforms = self._uniforms(sampling)
         tokens = self.sampler.sample(logits, temperatures, uniforms)
         rows = logits.cpu() if record_logits else None
         out, k = [], 0
@@ -69,6 +75,6 @@ class ModelExecutor:
         logits = self.runner.run(entries, (previous.tokens.on_device, pairs) if pairs else None)
         sampling = [w for w in work if w.samples]
         temperatures = [w.seq.request.temperature for w in sampling]
-        uniforms = [uniform_for(w.seq.request.seed, w.seq.request_id, len(w.seq.generated)) for w in sampling]
+        uniforms = self._uniforms(sampling)
         tokens = self.sampler.sample_on_device(logits, temperatures, uniforms)
         return LaunchedStep(tokens, {id(w.seq): k for k, w in enumerate(sampling)}, sampling)

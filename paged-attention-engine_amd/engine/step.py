@@ -148,6 +148,8 @@ class StepRunner:
             captured = self._graphs.get(key)
             if captured is None:
                 if len(self._graphs) >= self.MAX_GRAPHS:
+                    # the oldest recording goes; a step launched from it may still be running
+                    torch.cuda.current_stream().synchronize()
                     self._graphs.pop(next(iter(self._graphs)))
                 captured = self._graphs[key] = _CapturedStep(torch.empty(len(flat), dtype=torch.int32,
                                                                          device=self.device))
