@@ -11,8 +11,8 @@
 // order: no atomics, the same sums in the same order on every run.
 //
 // Epilogues: bfloat16 out with bias; float32 out (logits, or partial sums);
-// SiLU gate: rows come in blocks of 16 gate rows followed by their 16 up rows,
-// and out[m, j] = silu(gate_j) * up_j (engine/model.py:317-320 of the reference);
+// SiLU gate: rows come in blocks of 8 gate rows followed by their 8 up rows (one tile of the
+// matrix instruction holds both), and out[m, j] = silu(gate_j) * up_j (engine/model.py:317-320 of the reference);
 // rotation: W holds the query, key and value projections of an attention layer, a
 // tile takes 8 features of a head and the 8 they are rotated with, queries come out
 // rotated and keys and values go straight to their cache slots (engine/model.py:
@@ -136,17 +136,19 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
     const int m = 16 * mt + r;
     if (m >= M) continue;
     if (EPI == EPI_SWIGLU) {
+      // a tile holds 8 gate rows (lanes 0-31: rows 4 g4 + i) and their 8 up rows (lanes 32-63, same m)
 #pragma unroll
-      for (int pair = 0; pair < RT / 2; ++pair) {  // tiles 2 pair (gate) and 2 pair + 1 (up)
-        const int j = (tile_base / 2 + pair) * 16 + 4 * g4;  // output feature of register 0
-        if (j >= N / 2) continue;                                    // N counts gate and up rows
+      for (int rt = 0; rt < RT; ++rt) {
+        const int j = (tile_base + rt) * 8 + 4 * (g4 % 2);  // output feature of register 0
         s16x4 v;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float g = acc[2 * pair][mt][i], u = acc[2 * pair + 1][mt][i];
-          v[i] = to_bf16_bits(g / (1.0f + expf(-g)) * u);
+          const float own = acc[rt][mt][i];
+          const float up = __shfl_xor(own, 32);  // in every lane
+          v[i] = to_bf16_bits(own / (1.0f + expf(-own)) * up);
         }
-        *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j) = v;
+        if (g4 < 2 && j < N / 2)  // N counts gate and up rows
+          *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j) = v;
       }
     } else {
 #pragma unroll
@@ -188,7 +190,6 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
                                                           const void* __restrict__ bias, int b_is_f32, int M,
                                                           int N, int K, int k_per_split, int64_t part_stride,
                                                           SkinnyRope rope) {
-  static_assert(EPI != EPI_SWIGLU || RT % 2 == 0, "the gated epilogue pairs a gate tile with its up tile");
   __shared__ float s_part[MT == 1 ? 3 : 4][RT * MT * 4][PAE_WAVE];
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
@@ -445,7 +446,7 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
 
 // epilogue: 0 bfloat16 out (+bias), 1 float32 out (`splits` partials of `part_stride`
 // elements each when splits > 1; a bias only with one split), 2 SiLU gate (N counts the
-// interleaved gate and up rows; out is [M, N / 2]).
+// interleaved gate and up rows, 8 and 8; out is [M, N / 2]).
 static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
                          const void* bias, int b_is_f32, int M, int N, int K, int splits, int64_t part_stride,
                          const SkinnyRope& rope, hipStream_t stream) {
@@ -454,11 +455,11 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
               N, K, (long long)lda);
   PAE_REQUIRE(splits >= 1 && (splits == 1 || epilogue == EPI_F32), "gemm_skinny: %d k ranges need the float32 epilogue", splits);
   PAE_REQUIRE(!(bias && splits > 1), "gemm_skinny: a bias cannot be combined with partial sums");
-  PAE_REQUIRE(epilogue != EPI_SWIGLU || (N % 32 == 0 && ldc % 4 == 0), "gemm_skinny: gated epilogue needs N %% 32 == 0, got %d", N);
+  PAE_REQUIRE(epilogue != EPI_SWIGLU || (N % 16 == 0 && ldc % 4 == 0), "gemm_skinny: gated epilogue needs N %% 16 == 0, got %d", N);
   if (M == 0) return 0;
   // weight rows per workgroup: 16 for up to 16 rows of A, else 32 (see the kernel)
   const int mt = (M + 15) / 16;
-  const int rt = (mt >= 2 || epilogue == EPI_SWIGLU) ? 2 : 1;
+  const int rt = mt >= 2 ? 2 : 1;
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + 127) / 128 * 128;
   PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "gemm_skinny: %d k ranges are too many for K=%d", splits, K);
@@ -494,7 +495,7 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
                                                                bias, b_is_f32, M, N, K, k_per_split, part_stride, rope)
 #define BY_MT(EPI)                                                   \
   switch (mt) {                                                      \
-    case 1: LAUNCH(1, (EPI == EPI_SWIGLU ? 2 : 1), EPI); break;       \
+    case 1: LAUNCH(1, 1, EPI); break;                                \
     case 2: LAUNCH(2, 2, EPI); break;                                \
     case 3: LAUNCH(3, 2, EPI); break;                                \
     default: LAUNCH(4, 2, EPI); break;                               \

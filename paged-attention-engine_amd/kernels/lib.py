@@ -258,7 +258,7 @@ def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optio
     """out = a @ w^T for at most 64 rows of `a`, reading `w` once.
 
     EPI_BF16: out [M, N] bfloat16 (+bias).  EPI_F32: out [M, N] float32, or [splits, M, N]
-    partial sums over k ranges.  EPI_SWIGLU: w holds blocks of 16 gate rows followed by their 16
+    partial sums over k ranges.  EPI_SWIGLU: w holds blocks of 8 gate rows followed by their 8
     up rows; out [M, N / 2] = silu(gate) * up."""
     _gpu(out, a, w, bias)
     M, K_ = a.shape

@@ -28,7 +28,7 @@ class SwiGLU(Part):
                 prefix + "up_proj.weight": (s.intermediate_size, s.hidden_size),
                 prefix + "down_proj.weight": (s.hidden_size, s.intermediate_size)}
 
-    BLOCK = 16  # gate and up rows alternate in blocks of this many (the skinny product's gated epilogue)
+    BLOCK = 8  # gate and up rows alternate in blocks of this many (the skinny product's gated epilogue)
 
     def bind(self, prefix, weights):
         gate, up = weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]

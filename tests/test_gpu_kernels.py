@@ -145,21 +145,21 @@ def test_gemm_many_weight_rows(M, N, K_):
 
 
 @pytest.mark.parametrize("M", [1, 8, 33, 64])
-@pytest.mark.parametrize("inter,K_", [(8960, 1536), (176, 64), (48, 72)])
+@pytest.mark.parametrize("inter,K_", [(8960, 1536), (176, 64), (48, 72), (40, 72), (37888, 136)])
 def test_gemm_skinny_gated(M, inter, K_):
     torch.manual_seed(inter)
     a = torch.randn(M, K_).to(torch.bfloat16)
     gate = (torch.randn(inter, K_) * 0.2).to(torch.bfloat16)
     up = (torch.randn(inter, K_) * 0.2).to(torch.bfloat16)
     want = plain.silu(a.double() @ gate.double().t()) * (a.double() @ up.double().t())
-    w = torch.stack([gate.view(inter // 16, 16, K_), up.view(inter // 16, 16, K_)], dim=1).reshape(2 * inter, K_)
+    w = torch.stack([gate.view(inter // 8, 8, K_), up.view(inter // 8, 8, K_)], dim=1).reshape(2 * inter, K_)
     out = torch.empty(M, inter, dtype=torch.bfloat16, device=DEV)
     K().gemm_skinny(out, a.to(DEV), w.contiguous().to(DEV), None, K().EPI_SWIGLU)
     assert (out.double().cpu() - want).abs().max() <= 2.0 ** -7 * float(want.abs().max())
     # the separate gate kernel reads the same interleaved layout
     both = (a.double() @ w.double().t()).to(torch.bfloat16)
     out2 = torch.empty(M, inter, dtype=torch.bfloat16, device=DEV)
-    K().swiglu(out2, both.to(DEV), 16)
+    K().swiglu(out2, both.to(DEV), 8)
     assert (out2.double().cpu() - want).abs().max() <= 2.0 ** -6 * float(want.abs().max())
 
 
