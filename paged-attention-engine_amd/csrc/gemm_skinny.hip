@@ -334,20 +334,20 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
 
 // The same product for 17..64 rows of A where there are many weight rows.  With several column
 // tiles the kernel above is held up by the activations, which every workgroup reads again for its
-// few weight rows, and by adding up its four wavefronts' sums.  Here a workgroup takes 128 weight
-// rows, 32 per wavefront over the whole k range, and reads each 128-wide slab of the activations
-// once: all threads load it together and leave it in LDS in the order the matrix instruction
+// few weight rows, and by adding up its four wavefronts' sums.  Here a workgroup takes 64 RT weight
+// rows, 16 RT per wavefront over the whole k range, and reads each slab of the activations (128 wide
+// with RT = 2, 256 wide with RT = 1: the same weight bytes on their way) once: all threads load it together and leave it in LDS in the order the matrix instruction
 // wants, where every wavefront reads its fragments with one 16-byte read each (two slabs take
 // turns: the next is fetched while the current one is used).  Weight fragments come straight
 // from memory as above.  Every wavefront ends with whole sums of its own rows.
-template <int MT, int EPI>
+template <int MT, int RT, int EPI>
 __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out, int64_t ldc,
                                                           const bf16_t* __restrict__ A, int64_t lda,
                                                           const bf16_t* __restrict__ W,
                                                           const void* __restrict__ bias, int b_is_f32, int M,
                                                           int N, int K, int k_per_split, int64_t part_stride,
                                                           SkinnyRope rope) {
-  constexpr int RT = 2, KC = 128;
+  constexpr int KC = 256 / RT, CH = KC / 128;
   __shared__ bf16x8 a_lds[2][MT][KC / 32][PAE_WAVE];  // [slab][column tile][k step][lane]
   const int tid = threadIdx.x, lane = tid % PAE_WAVE, wave = tid / PAE_WAVE;
   const int g4 = lane / 16;
@@ -384,12 +384,15 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
     for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {};
   struct Slab {
-    bf16x8 wf[KC / 32][RT], a[MT];
+    bf16x8 wf[KC / 32][RT], a[MT][CH];
   };
   auto load = [&](Slab& b, int kc) {  // loads are unconditional, from clamped addresses
-    const int ka = kc + 8 * achunk;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) b.a[mt] = *reinterpret_cast<const bf16x8*>(aptr[mt] + (ka < K - 8 ? ka : K - 8));
+    for (int c = 0; c < CH; ++c) {
+      const int ka = kc + 128 * c + 8 * achunk;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) b.a[mt][c] = *reinterpret_cast<const bf16x8*>(aptr[mt] + (ka < K - 8 ? ka : K - 8));
+    }
 #pragma unroll
     for (int st = 0; st < KC / 32; ++st) {
       const int k = kc + 32 * st + 8 * lkg;
@@ -399,7 +402,9 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
   };
   auto stage = [&](const Slab& b, int buf) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) a_lds[buf][mt][a_step][a_slot] = b.a[mt];
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int c = 0; c < CH; ++c) a_lds[buf][mt][4 * c + a_step][a_slot] = b.a[mt][c];
   };
   auto multiply = [&](Slab& b, int kc, int buf) {
 #pragma unroll
@@ -466,11 +471,20 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   // many weight rows and more than 16 rows of A: 128 weight rows a workgroup, activations through LDS
   // (measured at 1.5B/7B/72B layer sizes: ahead from about one workgroup per compute unit on, behind below)
   const int medium_groups = (N + 127) / 128;
+  // Up to 48 rows of A and fewer than four such workgroups per compute unit: 64 weight rows a workgroup
+  // instead (gate/up of the 7B sizes at 32 rows: 77 -> 61 us; at 64 rows the activations' re-reading costs
+  // more than the idle units, and with few weight rows, as at the 1.5B sizes, the first kernel stays ahead).
+  const int narrow_groups = (N + 63) / 64;
+  const bool wide = mt > 3 || (int64_t)medium_groups * splits >= 1024 || (int64_t)narrow_groups * splits < 512;
   if (mt >= 2 && (int64_t)medium_groups * splits >= 256) {
-    dim3 mgrid(medium_groups, splits);
-#define LAUNCH_MEDIUM(MT, EPI)                                                                                  \
-  gemm_medium_kernel<MT, EPI><<<mgrid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, bias, \
-                                                         b_is_f32, M, N, K, k_per_split, part_stride, rope)
+    dim3 mgrid(wide ? medium_groups : (N + 63) / 64, splits);
+#define LAUNCH_MEDIUM(MT, EPI)                                                                                   \
+  if (wide)                                                                                                      \
+    gemm_medium_kernel<MT, 2, EPI><<<mgrid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W,  \
+                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope); \
+  else                                                                                                           \
+    gemm_medium_kernel<MT, 1, EPI><<<mgrid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W,  \
+                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope)
 #define MEDIUM_BY_MT(EPI)                       \
   switch (mt) {                                 \
     case 2: LAUNCH_MEDIUM(2, EPI); break;       \
