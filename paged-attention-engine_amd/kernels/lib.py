@@ -249,6 +249,15 @@ def skinny_splits(N: int, K: int, M: int = 1) -> int:
     rows = 32 if M > 16 else 16
     tiles = -(-N // rows)
     wanted = max(1, min(512 // tiles, K // 256, 8))
+    if M > 16:
+        # enough ranges of at least 1024 for the many-weight-rows kernel (128 rows a workgroup) to fill
+        # the chip twice, where that many exist (72B down at 64 rows: 2 ranges 177 us, 8 ranges 115 us)
+        groups = -(-N // 128)
+        many = min(12, -(-512 // groups))
+        while many > 1 and K // many < 1024:
+            many -= 1
+        if groups * many >= 256:
+            wanted = max(wanted, many)
     k_per = -(-(-(-K // wanted)) // 128) * 128
     return -(-K // k_per)
 
