@@ -26,11 +26,14 @@ int pae_gemm_plain(int in_dtype, int out_dtype, void* C, int64_t ldc, const void
                    const void* bias, int b_is_f32, int M, int N, int K, hipStream_t stream);
 int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
                     const void* bias, int b_is_f32, int M, int N, int K, int splits, int64_t part_stride,
-                    hipStream_t stream);
+                    float* ticket_parts, int* ticket_counters, hipStream_t stream);
+int pae_skinny_ticket_slots(int M, int N);
+int64_t pae_skinny_ticket_floats(int M, int N, int splits);
 int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int64_t lda, const void* W, const void* bias,
                          int b_is_f32, int M, int K, int nh, int nkv, int hd, int rot, const float* cos_sin,
                          const int* positions, const int* tok_seq, const int* block_tables, int max_blocks, int bs,
-                         void* k_cache, void* v_cache, hipStream_t stream);
+                         void* k_cache, void* v_cache, int splits, float* ticket_parts, int* ticket_counters,
+                         hipStream_t stream);
 int pae_paged_attention_generic(int dtype, void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                 const void* k_cache, const void* v_cache, const int* positions,
                                 const int* tok_seq, const int* block_tables, int max_blocks, int bs,

@@ -179,6 +179,52 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
   }
 }
 
+// Several k ranges for an epilogue that needs whole sums (bias, rotation, gate): every range's
+// workgroup leaves its partial tile in `parts` and draws a ticket from the tile's counter; the one
+// that draws the last ticket knows that all partials are written, adds them in range order
+// whichever workgroup it is (so the sums do not depend on the order of arrival), puts the counter
+// back to zero and runs the epilogue.  Nobody waits for anybody.
+//
+// Workgroups run on several dies, each with an L2 of its own, so the partials are written and read
+// as device-scope atomic accesses, which go past the caches to memory, and a workgroup draws its
+// ticket only when its stores have been acknowledged.  (Ordinary stores followed by a device-scope
+// fence do the same, but the fence writes back the die's whole L2: measured at 13 us a launch.)
+struct SkinnyTickets {
+  float* parts;   // [slots][k ranges][RT * 4][64]: a wavefront's accumulators, lane by lane
+  int* counters;  // [slots], zero before and after every launch; null: one k range
+};
+
+// True in the wavefront that holds the whole sums afterwards (in `acc`); the others are done.
+template <int RT>
+__device__ __forceinline__ bool add_up_k_ranges(f32x4 (&acc)[RT], int slot, int split, int splits,
+                                                const SkinnyTickets& tk) {
+  const int lane = threadIdx.x % PAE_WAVE;
+  float* mine = tk.parts + ((int64_t)slot * splits + split) * (RT * 4 * PAE_WAVE) + lane;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __hip_atomic_store(mine + (rt * 4 + i) * PAE_WAVE, acc[rt][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every lane's stores have arrived
+  int ticket = 0;
+  if (lane == 0) ticket = __hip_atomic_fetch_add(tk.counters + slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  ticket = __builtin_amdgcn_readfirstlane(ticket);
+  asm volatile("" ::: "memory");
+  if (ticket != splits - 1) return false;  // the same in every lane
+  if (lane == 0) __hip_atomic_store(tk.counters + slot, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) acc[rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int p = 0; p < splits; ++p) {
+    const float* theirs = tk.parts + ((int64_t)slot * splits + p) * (RT * 4 * PAE_WAVE) + lane;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc[rt][i] += __hip_atomic_load(theirs + (rt * 4 + i) * PAE_WAVE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  return true;
+}
+
 // MT: column tiles of 16 rows of A; RT: tiles of 16 weight rows per workgroup; SKINNY_U: k steps
 // of a wavefront whose loads are in flight together.  With more
 // rows of A a workgroup takes more weight rows, so that the activations, which every
@@ -189,7 +235,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
                                                           const bf16_t* __restrict__ W,
                                                           const void* __restrict__ bias, int b_is_f32, int M,
                                                           int N, int K, int k_per_split, int64_t part_stride,
-                                                          SkinnyRope rope) {
+                                                          SkinnyRope rope, SkinnyTickets tickets) {
   __shared__ float s_part[MT == 1 ? 3 : 4][RT * MT * 4][PAE_WAVE];
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
@@ -328,6 +374,20 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
       }
   }
 
+  if (EPI != EPI_F32 && tickets.counters) {  // this wavefront's column tile: the sums of all k ranges, or done
+    f32x4 mine[RT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      if (MT == 1 || mt == wave)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) mine[rt] = acc[rt][mt];
+    if (!add_up_k_ranges<RT>(mine, blockIdx.x * MT + (MT > 1 ? wave : 0), blockIdx.y, gridDim.y, tickets)) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      if (MT == 1 || mt == wave)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) acc[rt][mt] = mine[rt];
+  }
   skinny_epilogue<MT, RT, EPI>(acc, blockIdx.x * RT, MT > 1 ? wave : -1, out, ldc, bias, b_is_f32, M, N, blockIdx.y,
                                part_stride, rope);
 }
@@ -346,7 +406,7 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
                                                           const bf16_t* __restrict__ W,
                                                           const void* __restrict__ bias, int b_is_f32, int M,
                                                           int N, int K, int k_per_split, int64_t part_stride,
-                                                          SkinnyRope rope) {
+                                                          SkinnyRope rope, SkinnyTickets tickets) {
   constexpr int KC = 256 / RT, CH = KC / 128;
   __shared__ bf16x8 a_lds[2][MT][KC / 32][PAE_WAVE];  // [slab][column tile][k step][lane]
   const int tid = threadIdx.x, lane = tid % PAE_WAVE, wave = tid / PAE_WAVE;
@@ -446,6 +506,11 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
     __syncthreads();
     kc += KC;
   }
+  if (EPI != EPI_F32 && tickets.counters) {  // this wavefront's rows: the sums of all k ranges, or done
+    if (!add_up_k_ranges<RT * MT>(reinterpret_cast<f32x4(&)[RT * MT]>(acc), blockIdx.x * 4 + wave, blockIdx.y,
+                                  gridDim.y, tickets))
+      return;
+  }
   skinny_epilogue<MT, RT, EPI>(acc, tile_base, -1, out, ldc, bias, b_is_f32, M, N, blockIdx.y, part_stride, rope);
 }
 
@@ -454,12 +519,15 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
 // interleaved gate and up rows, 8 and 8; out is [M, N / 2]).
 static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
                          const void* bias, int b_is_f32, int M, int N, int K, int splits, int64_t part_stride,
-                         const SkinnyRope& rope, hipStream_t stream) {
+                         const SkinnyRope& rope, SkinnyTickets tickets, hipStream_t stream) {
   PAE_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d is outside 0..64", M);
   PAE_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && lda % 8 == 0, "gemm_skinny: N=%d K=%d lda=%lld (K and lda must be multiples of 8)",
               N, K, (long long)lda);
-  PAE_REQUIRE(splits >= 1 && (splits == 1 || epilogue == EPI_F32), "gemm_skinny: %d k ranges need the float32 epilogue", splits);
-  PAE_REQUIRE(!(bias && splits > 1), "gemm_skinny: a bias cannot be combined with partial sums");
+  const bool ticketed = splits > 1 && epilogue != EPI_F32;
+  PAE_REQUIRE(splits >= 1 && (!ticketed || (tickets.parts && tickets.counters)),
+              "gemm_skinny: %d k ranges with epilogue %d need scratch for partial sums and tickets", splits, epilogue);
+  PAE_REQUIRE(!(bias && splits > 1 && !ticketed), "gemm_skinny: a bias cannot be combined with partial sums");
+  if (!ticketed) tickets = SkinnyTickets{nullptr, nullptr};
   PAE_REQUIRE(epilogue != EPI_SWIGLU || (N % 16 == 0 && ldc % 4 == 0), "gemm_skinny: gated epilogue needs N %% 16 == 0, got %d", N);
   if (M == 0) return 0;
   // weight rows per workgroup: 16 for up to 16 rows of A, else 32 (see the kernel)
@@ -481,10 +549,10 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
 #define LAUNCH_MEDIUM(MT, EPI)                                                                                   \
   if (wide)                                                                                                      \
     gemm_medium_kernel<MT, 2, EPI><<<mgrid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W,  \
-                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope); \
+                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets); \
   else                                                                                                           \
     gemm_medium_kernel<MT, 1, EPI><<<mgrid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W,  \
-                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope)
+                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets)
 #define MEDIUM_BY_MT(EPI)                       \
   switch (mt) {                                 \
     case 2: LAUNCH_MEDIUM(2, EPI); break;       \
@@ -506,7 +574,7 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   // four k steps of loads in flight per wavefront: deeper prefetch costs registers and measured slower
 #define LAUNCH(MT, RT, EPI)                                                                                  \
   gemm_skinny_kernel<MT, RT, EPI, (MT == 1 ? 4 : 2)><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
-                                                               bias, b_is_f32, M, N, K, k_per_split, part_stride, rope)
+                                                               bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets)
 #define BY_MT(EPI)                                                   \
   switch (mt) {                                                      \
     case 1: LAUNCH(1, 1, EPI); break;                                \
@@ -526,12 +594,24 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   return pae_check_launch("gemm_skinny");
 }
 
+// Several k ranges with an epilogue other than float32 partial sums are added up inside the kernel:
+// ticket_parts is scratch of pae_skinny_ticket_floats(M, N, splits) floats and ticket_counters holds
+// pae_skinny_ticket_slots(M, N) ints that are zero before the call and zero after it.  Launches that
+// share the counters must not overlap.
 extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
                                const void* bias, int b_is_f32, int M, int N, int K, int splits,
-                               int64_t part_stride, hipStream_t stream) {
+                               int64_t part_stride, float* ticket_parts, int* ticket_counters, hipStream_t stream) {
   PAE_REQUIRE(epilogue != EPI_ROPE, "gemm_skinny: the rotating epilogue has an entry point of its own");
   return launch_skinny(epilogue, out, ldc, A, lda, W, bias, b_is_f32, M, N, K, splits, part_stride, SkinnyRope{},
-                       stream);
+                       SkinnyTickets{ticket_parts, ticket_counters}, stream);
+}
+
+// Counters and scratch floats that `splits` k ranges of an [M, K] x [N, K]^T product need for their
+// tickets, whichever kernel takes the product (one counter per wavefront that ends with whole sums of
+// its own; its accumulators for every range).
+extern "C" int pae_skinny_ticket_slots(int M, int N) { return (N + 15) / 16 * ((M + 15) / 16); }
+extern "C" int64_t pae_skinny_ticket_floats(int M, int N, int splits) {
+  return (int64_t)((N + 127) / 128) * 8 * ((M + 15) / 16) * splits * 4 * PAE_WAVE;
 }
 
 // q_out[M, nh * hd] = rotated queries of A * W^T (+ bias), W = [(nh + 2 nkv) * hd, K] holding the
@@ -543,7 +623,7 @@ extern "C" int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int
                                     const void* bias, int b_is_f32, int M, int K, int nh, int nkv, int hd, int rot,
                                     const float* cos_sin, const int* positions, const int* tok_seq,
                                     const int* block_tables, int max_blocks, int bs, void* k_cache, void* v_cache,
-                                    hipStream_t stream) {
+                                    int splits, float* ticket_parts, int* ticket_counters, hipStream_t stream) {
   PAE_REQUIRE(nh > 0 && nkv >= 0 && hd > 0 && hd % 16 == 0, "gemm_skinny_rope: bad head sizes nh=%d nkv=%d hd=%d", nh, nkv, hd);
   PAE_REQUIRE(rot >= 0 && rot <= hd && rot % 16 == 0 && (rot == 0 || cos_sin),
               "gemm_skinny_rope: rotary_dim %d must be a multiple of 16 up to head_dim %d", rot, hd);
@@ -553,5 +633,6 @@ extern "C" int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int
               "gemm_skinny_rope: the cache write needs tables and pools");
   SkinnyRope rope{cos_sin, positions, tok_seq, block_tables, (bf16_t*)k_cache, (bf16_t*)v_cache,
                   nh, nkv, hd, rot, max_blocks, bs};
-  return launch_skinny(EPI_ROPE, q_out, ldq, A, lda, W, bias, b_is_f32, M, (nh + 2 * nkv) * hd, K, 1, 0, rope, stream);
+  return launch_skinny(EPI_ROPE, q_out, ldq, A, lda, W, bias, b_is_f32, M, (nh + 2 * nkv) * hd, K, splits, 0, rope,
+                       SkinnyTickets{ticket_parts, ticket_counters}, stream);
 }

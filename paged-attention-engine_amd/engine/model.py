@@ -69,6 +69,8 @@ class Model:
         for block in self.blocks:
             block.bind(weights)
         self.final_norm.bind(plan.final_norm_prefix, weights)
+        if self.dtype == torch.bfloat16:
+            K.skinny_tickets(self.device)  # made before any step is recorded as a graph
         if plan.head_name is None:
             self.head = Linear(self.embedding)  # tied: the same buffer, no second copy
         else:

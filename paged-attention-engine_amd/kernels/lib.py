@@ -58,8 +58,9 @@ def _declare(lib) -> None:
         "pae_rope_table": [P, P, P, I, I, P],
         "pae_rope_kv_write": [I, P, L, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P],
         "pae_swiglu": [I, P, P, I, I, I, P],
-        "pae_gemm_skinny": [I, P, L, P, L, P, P, I, I, I, I, I, L, P],
-        "pae_gemm_skinny_rope": [P, L, P, L, P, P, I, I, I, I, I, I, I, P, P, P, P, I, I, P, P, P],
+        "pae_gemm_skinny": [I, P, L, P, L, P, P, I, I, I, I, I, L, P, P, P],
+        "pae_gemm_skinny_rope": [P, L, P, L, P, P, I, I, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P, P, P],
+        "pae_skinny_ticket_slots": [I, I],
         "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "pae_sample": [P, P, L, P, P, I, I, P, P, P, P],
@@ -72,6 +73,8 @@ def _declare(lib) -> None:
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = c_int
+    lib.pae_skinny_ticket_floats.argtypes = [I, I, I]
+    lib.pae_skinny_ticket_floats.restype = c_int64
 
 
 def _check(code: int) -> None:
@@ -268,21 +271,65 @@ def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optio
 
     EPI_BF16: out [M, N] bfloat16 (+bias).  EPI_F32: out [M, N] float32, or [splits, M, N]
     partial sums over k ranges.  EPI_SWIGLU: w holds blocks of 8 gate rows followed by their 8
-    up rows; out [M, N / 2] = silu(gate) * up."""
+    up rows; out [M, N / 2] = silu(gate) * up.  With several k ranges the other epilogues'
+    partial sums are added up inside the kernel (see `skinny_tickets`)."""
     _gpu(out, a, w, bias)
     M, K_ = a.shape
     N = w.shape[0]
     assert skinny_supported(a, w) and w.shape == (N, K_) and w.is_contiguous() and out.is_contiguous()
     if epilogue == EPI_SWIGLU:
-        assert out.shape == (M, N // 2) and out.dtype == torch.bfloat16 and splits == 1 and bias is None
+        assert out.shape == (M, N // 2) and out.dtype == torch.bfloat16 and bias is None
     elif epilogue == EPI_F32:
         assert out.dtype == torch.float32
         assert tuple(out.shape) == ((M, N) if splits == 1 and out.dim() == 2 else (splits, M, N))
     else:
-        assert out.shape == (M, N) and out.dtype == torch.bfloat16 and splits == 1
+        assert out.shape == (M, N) and out.dtype == torch.bfloat16
     bp, bf = _param(bias)
+    parts, counters = _ticket_scratch(a.device, M, N, splits if epilogue != EPI_F32 else 1)
     _check(library().pae_gemm_skinny(epilogue, out.data_ptr(), out.stride(-2), a.data_ptr(), a.stride(0),
-                                     w.data_ptr(), bp, bf, M, N, K_, splits, M * N, _stream()))
+                                     w.data_ptr(), bp, bf, M, N, K_, splits, M * N, _ptr(parts), _ptr(counters),
+                                     _stream()))
+
+
+_TICKETS: dict = {}
+
+
+def skinny_tickets(device) -> torch.Tensor:
+    """The zeroed counters of products whose k ranges are added up inside the kernel (every launch
+    leaves them zero; launches on one device run one after the other and share them).  Made at the
+    first call for a device, which must not come while a graph records: a model asks when it is
+    bound."""
+    index = torch.device(device).index or 0
+    if index not in _TICKETS:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("the ticket counters must exist before a graph is recorded")
+        _TICKETS[index] = torch.zeros(1 << 16, dtype=torch.int32, device=device)
+    return _TICKETS[index]
+
+
+def _ticket_scratch(device, M: int, N: int, splits: int):
+    """(partial sums, counters) for a product whose k ranges are added up inside the kernel."""
+    if splits <= 1:
+        return None, None
+    lib, counters = library(), skinny_tickets(device)
+    if lib.pae_skinny_ticket_slots(M, N) > counters.numel():
+        raise KernelError(f"{N} weight rows by {M} rows need more ticket counters than there are")
+    return torch.empty(lib.pae_skinny_ticket_floats(M, N, splits), dtype=torch.float32, device=device), counters
+
+
+def whole_sum_splits(N: int, K: int, M: int) -> int:
+    """k ranges for a product whose epilogue needs whole sums (gate, rotation, bias), which the
+    kernel then adds up itself.  That costs a trip to memory, and pays where the many-weight-rows
+    kernel has little more than one workgroup per compute unit (gate/up of the 7B sizes at 64
+    rows: 85 -> 72 us; with fewer weight rows, or with many more, one range is faster)."""
+    groups = -(-N // 128)
+    if M <= 16 or not 256 <= groups < 384:
+        return 1
+    wanted = -(-(768 if M > 48 else 512) // groups)
+    if K // wanted < 512:
+        return 1
+    k_per = -(-(-(-K // wanted)) // 128) * 128
+    return -(-K // k_per)
 
 
 def skinny_rope_supported(a: torch.Tensor, w: torch.Tensor, hd: int, rot: int) -> bool:
@@ -294,7 +341,8 @@ def skinny_rope_supported(a: torch.Tensor, w: torch.Tensor, hd: int, rot: int) -
 def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], nh: int,
                      nkv: int, hd: int, rot: int, cos_sin: Optional[torch.Tensor], positions: torch.Tensor,
                      tok_seq: Optional[torch.Tensor], block_tables: Optional[torch.Tensor], block_size: int,
-                     k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor]) -> None:
+                     k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                     splits: Optional[int] = None) -> None:
     """Query/key/value projection of at most 64 rows with the rotation and the cache write in its
     epilogue: q_out[M, nh * hd] = rotated queries; rotated keys and raw values go to their slots
     (nkv == 0: `w` holds the query rows only and nothing is stored).  `cos_sin`: see `rope_table`."""
@@ -312,10 +360,14 @@ def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias
         _check_pools(k_cache, v_cache, nkv, block_size, hd)
         max_blocks = block_tables.shape[1]
     bp, bf = _param(bias)
-    _check(library().pae_gemm_skinny_rope(q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(),
-                                          bp, bf, M, K_, nh, nkv, hd, rot, _ptr(cos_sin) if rot else None,
-                                          positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks,
-                                          block_size, _ptr(k_cache), _ptr(v_cache), _stream()))
+    lib, N = library(), w.shape[0]
+    splits = 1 if splits is None else splits
+    parts, counters = _ticket_scratch(a.device, M, N, splits)
+    _check(lib.pae_gemm_skinny_rope(q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(),
+                                    bp, bf, M, K_, nh, nkv, hd, rot, _ptr(cos_sin) if rot else None,
+                                    positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks,
+                                    block_size, _ptr(k_cache), _ptr(v_cache), splits, _ptr(parts), _ptr(counters),
+                                    _stream()))
 
 
 def gemm_plain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:

@@ -46,7 +46,8 @@ class SwiGLU(Part):
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         act = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
         if self.block and x.shape[0] and K.skinny_supported(x, self.gate_up.weight):
-            K.gemm_skinny(act, x, self.gate_up.weight, None, K.EPI_SWIGLU)
+            splits = K.whole_sum_splits(2 * self.spec.intermediate_size, self.spec.hidden_size, x.shape[0])
+            K.gemm_skinny(act, x, self.gate_up.weight, None, K.EPI_SWIGLU, splits)
         else:
             K.swiglu(act, self.gate_up(x), self.block)
         return self.down.branch(act)

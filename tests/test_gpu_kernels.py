@@ -138,6 +138,13 @@ def test_gemm_many_weight_rows(M, N, K_):
     parts = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device=DEV)
     K().gemm_skinny(parts, d_a, d_w, None, K().EPI_F32, splits)
     assert (parts.sum(0).double().cpu() - want).abs().max() <= 2e-5 * scale
+    if K_ > 128:  # the bias epilogue over several k ranges: partial sums are added up inside the kernel
+        ranges = 4 if K_ >= 1024 else 2
+        for _ in range(2):  # the second call finds the tickets as the first left them
+            out_k = torch.full((M, N), 77.0, dtype=torch.bfloat16, device=DEV)
+            K().gemm_skinny(out_k, d_a, d_w, b.to(DEV), K().EPI_BF16, ranges)
+            assert int(K().skinny_tickets(DEV).abs().sum()) == 0
+            assert (out_k.double().cpu() - (want + b.double())).abs().max() <= 2.0 ** -7 * (scale + 3)
     # a row alone goes through the few-row kernel, which adds in another order: equal to rounding
     one = torch.empty(1, N, dtype=torch.float32, device=DEV)
     K().gemm_skinny(one, d_a[M - 1:], d_w, None, K().EPI_F32)
@@ -156,6 +163,13 @@ def test_gemm_skinny_gated(M, inter, K_):
     out = torch.empty(M, inter, dtype=torch.bfloat16, device=DEV)
     K().gemm_skinny(out, a.to(DEV), w.contiguous().to(DEV), None, K().EPI_SWIGLU)
     assert (out.double().cpu() - want).abs().max() <= 2.0 ** -7 * float(want.abs().max())
+    # several k ranges, added up inside the kernel (twice: the tickets are back at zero in between)
+    if K_ > 128:
+        for _ in range(2):
+            out_k = torch.full_like(out, 3.0)
+            K().gemm_skinny(out_k, a.to(DEV), w.contiguous().to(DEV), None, K().EPI_SWIGLU, min(3, -(-K_ // 128)))
+            assert int(K().skinny_tickets(DEV).abs().sum()) == 0
+            assert (out_k.double().cpu() - want).abs().max() <= 2.0 ** -7 * float(want.abs().max())
     # the separate gate kernel reads the same interleaved layout
     both = (a.double() @ w.double().t()).to(torch.bfloat16)
     out2 = torch.empty(M, inter, dtype=torch.bfloat16, device=DEV)
@@ -291,10 +305,13 @@ def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs):
 @pytest.mark.parametrize("nh,nkv,hd,rot,bs,Kdim,bias", [
     (4, 2, 16, 16, 4, 72, True), (6, 1, 48, 48, 16, 136, False), (3, 3, 32, 16, 8, 264, True),
     (5, 1, 64, 0, 16, 200, True), (12, 2, 128, 128, 16, 1536, True), (248, 4, 128, 64, 16, 136, True)])
-def test_gemm_skinny_rope(M, nh, nkv, hd, rot, bs, Kdim, bias):
+@pytest.mark.parametrize("k_ranges", ["one", "chosen", "several"])
+def test_gemm_skinny_rope(M, nh, nkv, hd, rot, bs, Kdim, bias, k_ranges):
     """The projection with rotation and cache write in its epilogue against: a float64 product,
-    rounded to bfloat16 (as the separate projection would), rotated, and laid into the pools."""
+    rounded to bfloat16 (as the separate projection would), rotated, and laid into the pools.
+    With several k ranges the kernel adds up its workgroups' partial sums itself."""
     torch.manual_seed(M + nh)
+    splits = {"one": 1, "chosen": None, "several": min(3, -(-Kdim // 128))}[k_ranges]
     theta = 50000.0
     # three sequences take turns; positions grow by 3 per row so that rows land in different pages
     tok_seq = [t % 3 for t in range(M)]
@@ -314,7 +331,8 @@ def test_gemm_skinny_rope(M, nh, nkv, hd, rot, bs, Kdim, bias):
            if rot else None)
     K().gemm_skinny_rope(q, a.to(DEV), w.to(DEV), None if b is None else b.to(DEV), nh, nkv, hd, rot, inv,
                          torch.tensor(positions, dtype=torch.int32, device=DEV),
-                         torch.tensor(tok_seq, dtype=torch.int32, device=DEV), tables.to(DEV), bs, d_kp, d_vp)
+                         torch.tensor(tok_seq, dtype=torch.int32, device=DEV), tables.to(DEV), bs, d_kp, d_vp, splits)
+    assert int(K().skinny_tickets(DEV).abs().sum()) == 0  # the tickets are back at zero
     exact = a.double() @ w.double().t() + (0 if b is None else b.double())
     x = exact.to(torch.bfloat16).double().view(M, nh + 2 * nkv, hd)
     rotated = x.clone()
@@ -340,9 +358,9 @@ def test_gemm_skinny_rope(M, nh, nkv, hd, rot, bs, Kdim, bias):
     q2 = torch.empty_like(q)
     K().gemm_skinny_rope(q2, a.to(DEV), w[:nh * hd].contiguous().to(DEV), None if b is None else b[:nh * hd].to(DEV),
                          nh, 0, hd, rot, inv, torch.tensor(positions, dtype=torch.int32, device=DEV), None, None, bs,
-                         None, None)
-    # (bit for bit where both calls take the same kernel; the many-row kernel adds in another order)
-    assert (q2.double() - q.double()).abs().max().item() <= (0.0 if N < 32768 else bound)
+                         None, None, splits)
+    # (bit for bit where both calls take the same kernel and k ranges; the many-row kernel adds in another order)
+    assert (q2.double() - q.double()).abs().max().item() <= (0.0 if N < 32768 and splits is not None else bound)
 
 
 # ------------------------------------------------------------------ attention
