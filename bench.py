@@ -180,7 +180,7 @@ def main() -> int:
     step_bytes = weight_bytes(cfg, elem) + kv_bytes(cfg, tokens_held, elem)
     achieved = step_bytes / step_s / 1e9
     record = {
-        "metric": "decode tok/s at batch 8, context 4096 (Qwen2.5-1.5B shape)",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.ctx} (Qwen2.5-1.5B shape)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",

@@ -237,6 +237,17 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
                                                           int N, int K, int k_per_split, int64_t part_stride,
                                                           SkinnyRope rope, SkinnyTickets tickets) {
   __shared__ float s_part[MT == 1 ? 3 : 4][RT * MT * 4][PAE_WAVE];
+  if (MT == 1 && gridDim.z > 1) {  // the rows of A are shared out in tiles of 16: this workgroup's tile
+    const int m0 = blockIdx.z * 16;
+    A += (int64_t)m0 * lda;
+    out = EPI == EPI_F32 ? (void*)((float*)out + (int64_t)m0 * ldc) : (void*)((bf16_t*)out + (int64_t)m0 * ldc);
+    M = min(16, M - m0);
+    if (EPI == EPI_ROPE) {
+      rope.positions += m0;
+      if (rope.tok_seq) rope.tok_seq += m0;
+      if (rope.cos_sin) rope.cos_sin += (int64_t)m0 * rope.rot;
+    }
+  }
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
   const int n0 = blockIdx.x * 16 * RT;
@@ -569,6 +580,24 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
 #undef MEDIUM_BY_MT
 #undef LAUNCH_MEDIUM
     return pae_check_launch("gemm_medium");
+  }
+  // Very few weight rows (the QKV product of the 1.5B sizes: 64 workgroups of 32 rows): the rows of A are
+  // shared out too, 16 to a workgroup of the one-tile kernel, and the weights are read once from HBM and
+  // again from L2 (1.5B QKV at 64 rows 10.5 -> 6.7 us; from about 100 workgroups on it is slower).
+  if (mt >= 2 && !ticketed && (int64_t)((N + 31) / 32) * splits <= 96) {
+    dim3 tiled((N + 15) / 16, splits, mt);
+#define LAUNCH_TILED(EPI)                                                                                        \
+  gemm_skinny_kernel<1, 1, EPI, 4><<<tiled, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, bias, \
+                                                               b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets)
+    switch (epilogue) {
+      case EPI_BF16: LAUNCH_TILED(EPI_BF16); break;
+      case EPI_F32: LAUNCH_TILED(EPI_F32); break;
+      case EPI_SWIGLU: LAUNCH_TILED(EPI_SWIGLU); break;
+      case EPI_ROPE: LAUNCH_TILED(EPI_ROPE); break;
+      default: return pae_fail("gemm_skinny: unknown epilogue %d", epilogue);
+    }
+#undef LAUNCH_TILED
+    return pae_check_launch("gemm_skinny (rows of A in tiles)");
   }
   dim3 grid((N + 16 * rt - 1) / (16 * rt), splits);
   // four k steps of loads in flight per wavefront: deeper prefetch costs registers and measured slower
