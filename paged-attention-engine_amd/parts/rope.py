@@ -55,8 +55,9 @@ class NeoxRope(Part):
 
 def _fused_projection(rot, cos_sin, ctx, x, linear, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
     q = torch.empty((x.shape[0], nh * hd), dtype=x.dtype, device=x.device)
+    splits = K.whole_sum_splits(linear.out_features, linear.in_features, x.shape[0])
     K.gemm_skinny_rope(q, x, linear.weight, linear.bias, nh, nkv, hd, rot, cos_sin, ctx.positions, ctx.tok_seq,
-                       block_table, block_size, k_cache, v_cache)
+                       block_table, block_size, k_cache, v_cache, splits)
     return q
 
 
