@@ -261,6 +261,11 @@ def skinny_splits(N: int, K: int, M: int = 1) -> int:
             many -= 1
         if groups * many >= 256:
             wanted = max(wanted, many)
+        # or fewer, longer ranges for that kernel's 64-row workgroups, where those fill the chip and the
+        # 128-row ones do not (7B down at 48 rows: 12 ranges 47 us, 8 ranges of 64-row workgroups 42 us)
+        fewer = -(-448 // -(-N // 64))
+        if fewer <= 8 and K // fewer >= 1024 and groups * fewer < 256:
+            wanted = fewer
     k_per = -(-(-(-K // wanted)) // 128) * 128
     return -(-K // k_per)
 
