@@ -151,6 +151,24 @@ def test_gemm_many_weight_rows(M, N, K_):
     assert (one[0] - out32[M - 1]).abs().max() <= 2e-5 * scale
 
 
+@pytest.mark.parametrize("M", [17, 48, 64])
+def test_gemm_partial_sums_on_small_workgroups(M):
+    """Weight rows too few for 128-row workgroups to fill the chip, enough k ranges for 64-row ones:
+    the float32 partial sums come from the many-weight-rows kernel's smaller workgroups."""
+    torch.manual_seed(M)
+    N, K_, ranges = 3584, 2048, 8
+    a = (torch.randn(M, K_) * 0.5).to(torch.bfloat16)
+    w = (torch.randn(N, K_) * 0.1).to(torch.bfloat16)
+    want = a.double() @ w.double().t()
+    parts = torch.full((ranges, M, N), float("nan"), dtype=torch.float32, device=DEV)
+    K().gemm_skinny(parts, a.to(DEV), w.to(DEV), None, K().EPI_F32, ranges)
+    assert (parts.sum(0).double().cpu() - want).abs().max() <= 2e-5 * float(want.abs().max())
+    # each range holds its own part of the sum
+    k_per = K_ // ranges
+    first = a[:, :k_per].double() @ w[:, :k_per].double().t()
+    assert (parts[0].double().cpu() - first).abs().max() <= 2e-5 * float(want.abs().max())
+
+
 @pytest.mark.parametrize("M", [1, 8, 33, 64])
 @pytest.mark.parametrize("inter,K_", [(8960, 1536), (176, 64), (48, 72), (40, 72), (37888, 136)])
 def test_gemm_skinny_gated(M, inter, K_):
