@@ -527,7 +527,10 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
 
 // epilogue: 0 bfloat16 out (+bias), 1 float32 out (`splits` partials of `part_stride`
 // elements each when splits > 1; a bias only with one split), 2 SiLU gate (N counts the
-// interleaved gate and up rows, 8 and 8; out is [M, N / 2]).
+// interleaved gate and up rows, 8 and 8; out is [M, N / 2]), 3 rotation and cache write.
+// Several k ranges of epilogues 0, 2 and 3 are added up inside the kernel (`tickets`).
+// Which kernel runs is decided here from the sizes alone, by rules measured at the layer
+// sizes of the 1.5B, 7B and 72B models.
 static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
                          const void* bias, int b_is_f32, int M, int N, int K, int splits, int64_t part_stride,
                          const SkinnyRope& rope, SkinnyTickets tickets, hipStream_t stream) {
