@@ -151,6 +151,31 @@ def test_gemm_many_weight_rows(M, N, K_):
     assert (one[0] - out32[M - 1]).abs().max() <= 2e-5 * scale
 
 
+def test_sums_over_k_ranges_inside_the_kernel_are_repeatable():
+    """Partial sums are added in range order whichever workgroup comes last, so a product gives the
+    same bits every time; two inputs take turns, so that a partial sum left over from the launch
+    before (or read before it was written) would show."""
+    torch.manual_seed(11)
+    M, inter, K_, ranges = 64, 18944, 1024, 3
+    w = (torch.randn(2 * inter, K_) * 0.05).to(torch.bfloat16).to(DEV)
+    inputs = [torch.randn(M, K_).to(torch.bfloat16).to(DEV) for _ in range(2)]
+    first = []
+    for a in inputs:
+        out = torch.empty(M, inter, dtype=torch.bfloat16, device=DEV)
+        K().gemm_skinny(out, a, w, None, K().EPI_SWIGLU, ranges)
+        first.append(out)
+    one_range = torch.empty(M, inter, dtype=torch.bfloat16, device=DEV)
+    K().gemm_skinny(one_range, inputs[0], w, None, K().EPI_SWIGLU)
+    assert (one_range.float() - first[0].float()).abs().max() <= 2.0 ** -6 * float(one_range.float().abs().max())
+    different = 0
+    for i in range(400):
+        out = torch.empty(M, inter, dtype=torch.bfloat16, device=DEV)
+        K().gemm_skinny(out, inputs[i % 2], w, None, K().EPI_SWIGLU, ranges)
+        different += int(not torch.equal(out, first[i % 2]))
+    assert different == 0
+    assert int(K().skinny_tickets(DEV).abs().sum()) == 0
+
+
 @pytest.mark.parametrize("M", [17, 48, 64])
 def test_gemm_partial_sums_on_small_workgroups(M):
     """Weight rows too few for 128-row workgroups to fill the chip, enough k ranges for 64-row ones:
