@@ -252,6 +252,10 @@ def skinny_splits(N: int, K: int, M: int = 1) -> int:
     rows = 32 if M > 16 else 16
     tiles = -(-N // rows)
     wanted = max(1, min(512 // tiles, K // 256, 8))
+    if M <= 16 and tiles >= 200 and tiles * wanted < 640 and K >= 4096:
+        # one or two workgroups per compute unit, each with a long way to go (14B down at 8 rows:
+        # 320 workgroups over 13,824 of k take 48 us with the norm, three ranges 35 us)
+        wanted = min(8, -(-960 // tiles))
     if M > 16:
         # enough ranges of at least 1024 for the many-weight-rows kernel (128 rows a workgroup) to fill
         # the chip twice, where that many exist (72B down at 64 rows: 2 ranges 177 us, 8 ranges 115 us)
