@@ -329,25 +329,21 @@ def _ticket_scratch(device, M: int, N: int, splits: int):
 def whole_sum_splits(N: int, K: int, M: int) -> int:
     """k ranges for a product whose epilogue needs whole sums (gate, rotation, bias), which the
     kernel then adds up itself.  That costs a trip to memory, and pays with more than 16 rows of
-    activations where workgroups are few (measured at the 1.5B, 7B and 72B layer sizes):
+    activations where workgroups are few (measured at the 1.5B to 72B layer sizes):
     * the many-weight-rows kernel with little more than one workgroup per compute unit (7B gate/up
-      at 64 rows: 85 -> 72 us; with many more weight rows one range is faster);
-    * weight rows too few for that kernel, which a few ranges bring in (72B QKV at 64 rows:
-      87 -> 54 us), or, failing that, two or three ranges of the few-rows kernel (7B QKV: 26 -> 22 us);
+      at 64 rows: 85 -> 72 us; with more weight rows, or somewhat fewer, one range is as fast or faster);
+    * few weight rows (the QKV products): ranges of about 1,280 (7B at 64 rows 26 -> 22 us in three,
+      14B 37 -> 31 us in four, 72B 87 -> 54 us in six);
     * not with very few weight rows, where the rows of activations are shared out instead."""
     tiles, groups = -(-N // 32), -(-N // 128)
-    if M <= 16 or tiles <= 96:
+    if M <= 16 or tiles <= 96 or 128 <= groups < 256 or groups >= 384:
         return 1
     if groups >= 256:
-        wanted = -(-(768 if M > 48 else 512) // groups) if groups < 384 else 1
+        wanted = -(-(768 if M > 48 else 512) // groups)
         if K // wanted < 512:
             return 1
     else:
-        wanted = -(-384 // groups)
-        if wanted > 6 or K // wanted < 1024:
-            wanted = max(1, min(3, 512 // tiles))
-            if K // wanted < 1024:
-                return 1
+        wanted = min(8, max(1, (K + 640) // 1280))
     k_per = -(-(-(-K // wanted)) // 128) * 128
     return -(-K // k_per)
 
