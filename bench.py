@@ -87,8 +87,11 @@ def decode_run(model, cfg, batch: int, ctx: int, steps: int, warmup: int, block_
 
     # Prompts run in portions of at most 2,048 tokens a step, so the first
     # sequences decode while the last still prefill; every sequence holds at
-    # least `ctx` tokens when the clock starts.
-    prompt_len = ctx - warmup - 1
+    # least `ctx` tokens when the clock starts.  The context passes `ctx` in the
+    # middle of the warm-up: a decode step is recorded anew when its block tables
+    # grow past a multiple of 64 pages (once per 1,024 tokens), and at a context
+    # of a power of two that recording would otherwise be the first timed step.
+    prompt_len = ctx - warmup // 2 - 1
     slack = batch * prompt_len // 2048 + 4
     max_new = warmup + steps + slack + 2
     blocks = batch * (-(-(prompt_len + max_new) // block_size) + 1) + 2
