@@ -208,3 +208,63 @@ extern "C" int pae_sample(int* tokens, const float* logits, int64_t ld, const fl
                                                          temperature, uniform, vocab, chunks);
   return pae_check_launch("sample");
 }
+
+// ---------------------------------------------------------------------------------------------
+// pae_sample_static: the same three kernels with their chunk results in a buffer that is part of
+// the library's image on every GPU, so that the call allocates nothing (see api.h).
+//
+// Layout of the buffer: PAE_SAMPLE_STATIC_SLOTS doubles (chunk sums), then as many floats (chunk
+// maxima), then as many ints (where each maximum first occurs).  A slot is one (row, chunk) pair.
+// Nothing in it has to start at zero: every slot that a call reads, the same call has written
+// before (maxima and places for every row, sums for the rows that sample), so what the call before
+// left does not matter.  Calls that overlap on one GPU (two streams, two threads) share the buffer
+// and race; callers run them one after the other.
+#include <mutex>
+
+#define PAE_SAMPLE_STATIC_BYTES (PAE_SAMPLE_STATIC_SLOTS * (sizeof(double) + sizeof(float) + sizeof(int)))
+#define PAE_MAX_DEVICES 64
+
+static __device__ __align__(256) unsigned char scratch[PAE_SAMPLE_STATIC_BYTES];
+
+// The buffer's address on each device.  In host code `scratch` is only a handle for the runtime's
+// symbol table: the address a kernel can use comes from hipGetSymbolAddress, once per device with
+// that device current, because each GPU holds its own copy at its own address.
+static void* g_scratch_of_device[PAE_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int scratch_on_current_device(void** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return pae_fail("sample_static: no current device: %s", hipGetErrorString(err));
+  PAE_REQUIRE(dev >= 0 && dev < PAE_MAX_DEVICES, "sample_static: device %d beyond the %d this library keeps track of",
+              dev, PAE_MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (!g_scratch_of_device[dev]) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !ptr)
+      return pae_fail("sample_static: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(err));
+    g_scratch_of_device[dev] = ptr;
+  }
+  *out = g_scratch_of_device[dev];
+  return 0;
+}
+
+extern "C" int pae_sample_static_slots() { return PAE_SAMPLE_STATIC_SLOTS; }
+
+extern "C" int pae_sample_static(int* tokens, const float* logits, int64_t ld, const float* temperature,
+                                 const float* uniform, int num_rows, int vocab, hipStream_t stream) {
+  PAE_REQUIRE(num_rows >= 0 && vocab > 0, "sample_static: bad sizes rows=%d V=%d", num_rows, vocab);
+  const int64_t slots = (int64_t)num_rows * pae_sample_chunks(vocab);
+  PAE_REQUIRE(slots <= PAE_SAMPLE_STATIC_SLOTS,
+              "sample_static: %d rows of %d logits need %lld chunk slots, the built-in buffer holds %d "
+              "(use pae_sample with a workspace of the caller's)",
+              num_rows, vocab, (long long)slots, PAE_SAMPLE_STATIC_SLOTS);
+  void* base = nullptr;
+  if (int code = scratch_on_current_device(&base)) return code;
+  double* chunk_sum = (double*)base;
+  float* chunk_max = (float*)(chunk_sum + PAE_SAMPLE_STATIC_SLOTS);
+  int* chunk_arg = (int*)(chunk_max + PAE_SAMPLE_STATIC_SLOTS);
+  return pae_sample(tokens, logits, ld, temperature, uniform, num_rows, vocab, chunk_max, chunk_arg, chunk_sum,
+                    stream);
+}

@@ -65,6 +65,8 @@ def _declare(lib) -> None:
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "pae_sample": [P, P, L, P, P, I, I, P, P, P, P],
         "pae_sample_chunks": [I],
+        "pae_sample_static": [P, P, L, P, P, I, I, P],
+        "pae_sample_static_slots": [],
         "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, P, P],
         "pae_attn_decode_split": [],
         "pae_attn_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
@@ -492,3 +494,19 @@ def sample(tokens: torch.Tensor, logits: torch.Tensor, temperature: Optional[tor
     _check(library().pae_sample(tokens.data_ptr(), logits.data_ptr(), logits.stride(0), _ptr(temperature),
                                 _ptr(uniform), R, V, chunk_max.data_ptr(), chunk_arg.data_ptr(),
                                 _ptr(chunk_sum), _stream()))
+
+
+def sample_static(tokens: torch.Tensor, logits: torch.Tensor, temperature: Optional[torch.Tensor],
+                  uniform: Optional[torch.Tensor]) -> None:
+    """`sample` without a workspace: the chunk results go to a buffer inside the library's image on
+    the GPU, so nothing is allocated here or there.  Rows times chunks beyond that buffer's slots
+    are refused; calls that overlap on one GPU race (they share the buffer)."""
+    _gpu(tokens, logits, temperature, uniform)
+    R, V = logits.shape
+    assert logits.dtype == torch.float32 and logits.stride(1) == 1
+    assert tokens.dtype == torch.int32 and tokens.numel() == R
+    for t in (temperature, uniform):
+        if t is not None:
+            assert t.dtype == torch.float32 and t.numel() == R
+    _check(library().pae_sample_static(tokens.data_ptr(), logits.data_ptr(), logits.stride(0), _ptr(temperature),
+                                       _ptr(uniform), R, V, _stream()))
