@@ -1,2 +1,3 @@
 from .allocator import HOLE, AllocResult, AllocStatus, BlockAllocator, BlockTable
-from .manager import CacheGroup, CacheManager, PagedSpec, StateSlots, StateSpec
+from .manager import (PAGE, CacheGroup, CacheManager, PagedSpec, PagedTensor, StateSlots, StateSpec, attention_pages,
+                      bytes_of_one_page_everywhere)

@@ -14,27 +14,75 @@ window has passed them (`release_passed`).  A reservation takes pages in every
 group or in none (the reference's all-or-nothing `append_tokens`,
 engine/cache.py:238-257, carried over to several pools).
 
-Pool layout of one group: [entry][K|V][block][kv head][block_size * head_dim]; the
-keys of one (block, head) are one contiguous tile [block_size][head_dim], the
-values one contiguous tile stored transposed, [head_dim][block_size], which is
-what the attention kernels' matrix-core operands want.
+What a page holds is the mixer's business: a `PagedSpec` lists named tensors, each
+with the shape of one page of it, in which `PAGE` stands for the page's token count.
+A group's pool is one tensor per name, [stop][block][*page shape].  The attention
+mixer declares keys [kv head][PAGE][head_dim] (the keys of one (block, head) are one
+contiguous tile) and values stored transposed, [kv head][head_dim][PAGE], which is
+what its matrix-core kernels' operands want (`attention_pages`); a mixer that caches
+one latent vector per token declares one tensor [PAGE][width], and the manager
+needs no change for it.
+
+Every pool has one page more than its allocator hands out, and the state tensors one
+slot more (`padding_page`, `padding_slot`): rows that a recorded step is padded with
+live there, where no sequence's data ever is.
 """
 
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Mapping, Optional, Sequence, Tuple
+from typing import Dict, List, Mapping, Optional, Sequence, Tuple, Union
 
 import torch
 
 from .allocator import AllocResult, AllocStatus, BlockAllocator
 
+PAGE = "page"  # in a page shape: the number of tokens a page holds
+
+
+@dataclass(frozen=True)
+class PagedTensor:
+    """One cached tensor: its name and the shape of one page of it (`PAGE` where the page's
+    token count goes, which must appear exactly once)."""
+
+    name: str
+    page_shape: Tuple[Union[int, str], ...]
+
+    def __post_init__(self) -> None:
+        if sum(1 for d in self.page_shape if d == PAGE) != 1:
+            raise ValueError(f"cached tensor '{self.name}': its page shape {self.page_shape} must name PAGE once")
+
+    def shape(self, block_size: int) -> Tuple[int, ...]:
+        return tuple(block_size if d == PAGE else int(d) for d in self.page_shape)
+
+    def elements_per_token(self) -> int:
+        count = 1
+        for d in self.page_shape:
+            count *= 1 if d == PAGE else int(d)
+        return count
+
 
 @dataclass(frozen=True)
 class PagedSpec:
-    num_kv_heads: int
-    head_dim: int
+    """What a mixer keeps per token: named tensors and, if it only looks back so far, a window."""
+
+    tensors: Tuple[PagedTensor, ...]
     window: Optional[int] = None
+
+    def __post_init__(self) -> None:
+        names = [t.name for t in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a paged spec needs tensors with distinct names, got {names}")
+
+    def elements_per_token(self) -> int:
+        return sum(t.elements_per_token() for t in self.tensors)
+
+
+def attention_pages(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> PagedSpec:
+    """Keys "k" [kv head][PAGE][head_dim] and values "v" [kv head][head_dim][PAGE] (transposed
+    within the page), as the attention kernels read them."""
+    return PagedSpec((PagedTensor("k", (num_kv_heads, PAGE, head_dim)),
+                      PagedTensor("v", (num_kv_heads, head_dim, PAGE))), window)
 
 
 @dataclass(frozen=True)
@@ -43,13 +91,20 @@ class StateSpec:
     dtype: torch.dtype = torch.float32
 
 
+def bytes_of_one_page_everywhere(paged: Sequence[Optional[PagedSpec]], block_size: int, dtype: torch.dtype) -> int:
+    """Bytes that one more page in every group's pool costs (all stops of all groups): what a
+    pool of N pages per group takes is N times this."""
+    elem = torch.empty((), dtype=dtype).element_size()
+    return sum(spec.elements_per_token() for spec in paged if spec is not None) * block_size * elem
+
+
 class CacheGroup:
     def __init__(self, index: int, spec: PagedSpec, entries: List[int], num_blocks: int, block_size: int):
         self.index = index
         self.spec = spec
         self.entries = entries
         self.allocator = BlockAllocator(num_blocks, block_size)
-        self.pool: Optional[torch.Tensor] = None
+        self.pools: Dict[str, torch.Tensor] = {}  # tensor name -> [stop][block][*page shape]
 
     def max_blocks_for(self, total_tokens: int, max_chunk: Optional[int]) -> int:
         """Most pages one sequence of `total_tokens` can hold at a time when it
@@ -126,37 +181,46 @@ class CacheManager:
         self._tokens: Dict[int, int] = {}
         if device is not None:
             for group in self.groups:
-                s = group.spec
-                group.pool = torch.zeros(
-                    (len(group.entries), 2, group.allocator.num_blocks, s.num_kv_heads, block_size, s.head_dim),
-                    dtype=dtype, device=device)
+                for t in group.spec.tensors:
+                    group.pools[t.name] = torch.zeros(
+                        (len(group.entries), group.allocator.num_blocks + 1, *t.shape(block_size)),
+                        dtype=dtype, device=device)
             for entry, spec in enumerate(states):
                 if spec is not None:
-                    self.state_tensors[entry] = torch.zeros((num_slots, *spec.shape), dtype=spec.dtype, device=device)
+                    self.state_tensors[entry] = torch.zeros((num_slots + 1, *spec.shape), dtype=spec.dtype,
+                                                            device=device)
 
     # ------------------------------------------------------------------ lookups
+    def padding_page(self, group: int) -> int:
+        """The page of a group's pool that its allocator never hands out."""
+        return self.groups[group].allocator.num_blocks
+
+    @property
+    def padding_slot(self) -> int:
+        return self.slots.num_slots
+
     def group_of(self, entry: int) -> Optional[int]:
         hit = self._group_of_entry.get(entry)
         return None if hit is None else hit[0]
 
-    def kv_of(self, entry: int) -> Tuple[torch.Tensor, torch.Tensor]:
-        """(keys, values) pools of a stop: keys [block][kv head][block_size][head_dim],
-        values [block][kv head][head_dim][block_size]."""
+    def pages_of(self, entry: int) -> Dict[str, torch.Tensor]:
+        """The cached tensors of a stop by name, each [block][*page shape]."""
         g, i = self._group_of_entry[entry]
-        pool = self.groups[g].pool
-        return pool[i, 0], pool[i, 1].view(pool.shape[2], pool.shape[3], pool.shape[5], pool.shape[4])
+        return {name: pool[i] for name, pool in self.groups[g].pools.items()}
+
+    def kv_of(self, entry: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(keys, values) of a stop whose mixer declared `attention_pages`: keys
+        [block][kv head][block_size][head_dim], values [block][kv head][head_dim][block_size]."""
+        pages = self.pages_of(entry)
+        return pages["k"], pages["v"]
 
     def state_of(self, entry: int) -> torch.Tensor:
         return self.state_tensors[entry]
 
     def storage_bytes(self) -> int:
-        total = 0
-        for group in self.groups:
-            s = group.spec
-            elem = torch.empty((), dtype=self.dtype).element_size()
-            total += (len(group.entries) * 2 * group.allocator.num_blocks * s.num_kv_heads * self.block_size
-                      * s.head_dim * elem)
-        return total
+        elem = torch.empty((), dtype=self.dtype).element_size()
+        return sum(len(g.entries) * g.allocator.num_blocks * self.block_size * g.spec.elements_per_token() * elem
+                   for g in self.groups)
 
     # ------------------------------------------------------------------ sequences
     def sequence_ids(self) -> Tuple[int, ...]:
@@ -188,6 +252,10 @@ class CacheManager:
 
     def block_table(self, group: int, seq_id: int) -> Tuple[int, ...]:
         return self.groups[group].allocator.block_table(seq_id)
+
+    def table_array(self, group: int, seq_id: int):
+        """The table itself as an array of int32, not a copy: for the step's staging buffer."""
+        return self.groups[group].allocator.table_array(seq_id)
 
     def can_reserve(self, seq_id: int, count: int, margin: int = 0) -> bool:
         return all(g.allocator.new_blocks_for(seq_id, count) + margin <= g.allocator.num_free

@@ -114,6 +114,11 @@ class ModelPlan:
     head_name: Optional[str]  # None: the head shares the embedding matrix
     final_norm_prefix: str
     max_positions: Optional[int] = None
+    # what some architectures do around the blocks (the reference's model does none of it:
+    # engine/model.py:401,453-455 gathers rows and multiplies by the head as they are)
+    embedding_scale: float = 1.0            # the gathered rows are multiplied by this
+    logit_scale: float = 1.0                # the logits are multiplied by this ...
+    logit_softcap: Optional[float] = None   # ... and then, with a cap c, become c * tanh(logits / c)
     extra: Mapping[str, Any] = field(default_factory=dict)
 
     def __post_init__(self) -> None:
@@ -124,6 +129,8 @@ class ModelPlan:
                 raise ConfigError(
                     f"schedule entry {i} reads the cache of entry {entry.cache_from}, "
                     "which is not an earlier entry")
+        if self.logit_softcap is not None and not self.logit_softcap > 0:
+            raise ConfigError(f"logit_softcap must be positive, got {self.logit_softcap}")
 
 
 def require(cfg: Mapping[str, Any], key: str, kind=int):

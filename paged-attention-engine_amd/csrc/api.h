@@ -10,7 +10,8 @@ const char* pae_last_error();
 int pae_device_arch(char* out, int cap);  // "gfx950" on the card the kernels are built for
 
 int pae_embedding(int dtype, void* out, const void* table, const int* ids, int num_tokens, int hidden,
-                  int vocab, hipStream_t stream);
+                  int vocab, float scale, hipStream_t stream);
+int pae_logits_finish(float* logits, int64_t n, float scale, float cap, hipStream_t stream);
 int pae_add_rmsnorm(int dtype, void* residual, const void* delta, int parts, int64_t part_stride,
                     const void* weight, int w_is_f32, float eps, const int* rows, void* out, int num_rows,
                     int hidden, int write_residual, hipStream_t stream);

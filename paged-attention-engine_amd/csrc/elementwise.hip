@@ -9,29 +9,48 @@
 #include "api.h"
 
 // ---------------------------------------------------------------- embedding
-// out[t, :] = table[ids[t], :]  (engine/model.py:401,448 of the reference: a plain
-// row gather, no scaling)
+// out[t, :] = scale * table[ids[t], :]  (engine/model.py:401,448 of the reference: a plain
+// row gather; its model has no scaling, so scale is 1 there and the product is exact)
 template <typename T>
 __global__ void embedding_kernel(float* __restrict__ out, const T* __restrict__ table,
-                                 const int* __restrict__ ids, int hidden) {
+                                 const int* __restrict__ ids, int hidden, float scale) {
   const int t = blockIdx.x;
   const T* row = table + (int64_t)ids[t] * hidden;
   float* dst = out + (int64_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(row[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = scale * to_f32(row[i]);
 }
 
 extern "C" int pae_embedding(int dtype, void* out, const void* table, const int* ids, int num_tokens,
-                             int hidden, int vocab, hipStream_t stream) {
+                             int hidden, int vocab, float scale, hipStream_t stream) {
   PAE_REQUIRE(num_tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes T=%d H=%d V=%d",
               num_tokens, hidden, vocab);
   if (num_tokens == 0) return 0;
   if (dtype == PAE_F32)
-    embedding_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)out, (const float*)table, ids, hidden);
+    embedding_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)out, (const float*)table, ids, hidden, scale);
   else if (dtype == PAE_BF16)
-    embedding_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((float*)out, (const bf16_t*)table, ids, hidden);
+    embedding_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((float*)out, (const bf16_t*)table, ids, hidden, scale);
   else
     return pae_fail("embedding: unknown dtype code %d", dtype);
   return pae_check_launch("embedding");
+}
+
+// ---------------------------------------------------------------- logits: scale and soft cap
+// x = scale * x, then, with cap > 0, x = cap * tanh(x / cap).  Not part of the reference's model
+// (its logits are the head product as it is); an architecture's plan may ask for either.
+__global__ void logits_finish_kernel(float* __restrict__ x, int64_t n, float scale, float cap) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float v = scale * x[i];
+  if (cap > 0.f) v = cap * tanhf(v / cap);
+  x[i] = v;
+}
+
+extern "C" int pae_logits_finish(float* logits, int64_t n, float scale, float cap, hipStream_t stream) {
+  PAE_REQUIRE(n >= 0 && n <= ((int64_t)1 << 38), "logits_finish: bad count %lld", (long long)n);
+  PAE_REQUIRE(cap >= 0.f, "logits_finish: the soft cap %g must not be negative (0 switches it off)", (double)cap);
+  if (n == 0) return 0;
+  logits_finish_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(logits, n, scale, cap);
+  return pae_check_launch("logits_finish");
 }
 
 // ---------------------------------------------------------------- add + RMSNorm

@@ -17,9 +17,9 @@ from typing import Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
-from ..config.engine_config import ADMISSION_MARGIN_BLOCKS, BLOCK_SIZE, NUM_GPU_BLOCKS, EngineConfig
+from ..config.engine_config import ADMISSION_MARGIN_BLOCKS, BLOCK_SIZE, EngineConfig
 from .executor import ModelExecutor
-from .model import Model, load_model
+from .model import TORCH_DTYPE, Model, load_model, random_model
 from .scheduler import EventKind, Request, Scheduler, StepResult
 
 
@@ -33,19 +33,38 @@ class GenerationResult:
 
 class Engine:
     def __init__(self, model: Union[str, Model], dtype: str = "bfloat16", block_size: int = BLOCK_SIZE,
-                 num_blocks: int = NUM_GPU_BLOCKS, max_num_seqs: Optional[int] = None,
+                 num_blocks: Optional[int] = None, max_num_seqs: Optional[int] = None,
                  max_num_batched_tokens: Optional[int] = None,
                  admission_margin_blocks: int = ADMISSION_MARGIN_BLOCKS, record_logits: bool = False,
-                 device: str = "cuda:0") -> None:
-        self.config = EngineConfig(dtype=dtype, block_size=block_size, num_blocks=num_blocks,
-                                   admission_margin_blocks=admission_margin_blocks,
+                 device: str = "cuda:0", kv_bytes: Optional[int] = None, fill_hbm: Optional[float] = None,
+                 num_state_slots: Optional[int] = None) -> None:
+        """`model`: a folder, or a built `Model`.  The pool: `num_blocks` pages in every cache
+        group (default 3,584), or `kv_bytes` for the whole cache, or `fill_hbm`, the share of
+        the device memory still free once the weights are in place."""
+        self.config = EngineConfig(dtype=dtype, block_size=block_size, num_blocks=num_blocks, kv_bytes=kv_bytes,
+                                   fill_hbm=fill_hbm, admission_margin_blocks=admission_margin_blocks,
                                    max_num_seqs=max_num_seqs, max_num_batched_tokens=max_num_batched_tokens,
-                                   device=device)
+                                   num_state_slots=num_state_slots, device=device)
         self.model = load_model(model, dtype, device) if isinstance(model, str) else model
-        self.cache = self.model.new_cache(block_size, num_blocks, self.config.state_slots)
+        if self.model.dtype != TORCH_DTYPE[dtype]:
+            raise ValueError(f"the engine was asked for {dtype} but the model it was given computes in {self.model.dtype}")
+        self.num_blocks = self.config.pages(self.model.page_bytes(block_size), self._free_device_bytes)
+        self.cache = self.model.new_cache(block_size, self.num_blocks, self.config.state_slots)
         self.executor = ModelExecutor(self.model, self.cache)
         self.record_logits = record_logits
         self.scheduler = self._new_scheduler()
+
+    @classmethod
+    def from_random(cls, config, seed: int = 0, dtype: str = "bfloat16", device: str = "cuda:0",
+                    std: float = 0.02, norm_std: float = 0.0, **engine_options) -> "Engine":
+        """An engine over random weights drawn on the device from `seed` (no folder is written);
+        `config` is a config.json dict or a typed config."""
+        return cls(random_model(config, seed, dtype, device, std, norm_std), dtype=dtype, device=device,
+                   **engine_options)
+
+    def _free_device_bytes(self) -> int:
+        torch.cuda.empty_cache()
+        return torch.cuda.mem_get_info(torch.device(self.config.device))[0]
 
     def _new_scheduler(self) -> Scheduler:
         c = self.config
@@ -56,9 +75,11 @@ class Engine:
 
     # the reference's scheduler surface
     def add_request(self, request: Union[Request, str], prompt_token_ids: Sequence[int] = (),
-                    max_new_tokens: int = 1, temperature: float = 0.0, seed: int = 0) -> bool:
+                    max_new_tokens: int = 1, temperature: float = 0.0, seed: int = 0,
+                    stop_token_ids: Sequence[int] = ()) -> bool:
         if not isinstance(request, Request):
-            request = Request(str(request), tuple(prompt_token_ids), max_new_tokens, temperature, seed)
+            request = Request(str(request), tuple(prompt_token_ids), max_new_tokens, temperature, seed,
+                              tuple(stop_token_ids))
         return self.scheduler.add_request(request)
 
     def step(self) -> StepResult:

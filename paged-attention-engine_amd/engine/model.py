@@ -16,14 +16,15 @@ from typing import Dict, List, Mapping, Optional, Tuple
 import torch
 
 from .. import models as _models  # noqa: F401  (registers the architectures)
-from ..cache.manager import CacheManager
+from ..cache.manager import CacheManager, bytes_of_one_page_everywhere
 from ..config.model_config import ModelPlan
-from ..config.registry import read_config
+from ..config.registry import read_config, read_config_dict
 from ..kernels import lib as K
 from ..parts import ResidualStream, StepContext, build_block, build_part
 from ..parts.base import NORMS
 from ..parts.linear import Linear
 from ..weights.loader import load_weights
+from ..weights.random_init import RandomWeights
 
 TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
@@ -77,18 +78,31 @@ class Model:
             self.head = Linear(weights[plan.head_name].to(device=self.device, dtype=self.dtype).contiguous())
 
     @property
+    def graph_max_rows(self) -> Optional[int]:
+        """Most rows a step may hold and still be recorded as a HIP graph (None: any number), as the
+        parts and the head's product say."""
+        limits = [block.graph_max_rows for block in self.blocks if block.graph_max_rows is not None]
+        if self.head is not None and self.head.graph_max_rows is not None:
+            limits.append(self.head.graph_max_rows)
+        return min(limits) if limits else None
+
+    @property
     def graph_safe(self) -> bool:
-        """Can a step of this model be recorded as a HIP graph?  Every part must launch
-        device work only, and every matrix product must go through this engine's own
-        kernels (library products may record memory clears into a graph)."""
+        """Can a step of this model be recorded as a HIP graph?  Every part must launch device
+        work from device-side data only, for some number of rows."""
         if not (all(block.graph_safe for block in self.blocks) and self.final_norm.graph_safe):
             return False
-        if self.dtype == torch.float32:
-            return True
-        widths = [self.plan.hidden_size]
+        return self.graph_max_rows is None or self.graph_max_rows > 0
+
+    def step_list_parts(self, block_size: int) -> Dict[object, object]:
+        """key -> the first part that asks for index lists under that key (see `Part.step_lists`)."""
+        out: Dict[object, object] = {}
         for block in self.blocks:
-            widths += getattr(block, "product_widths", lambda: [1])()
-        return all(w % 8 == 0 for w in widths)
+            for part in getattr(block, "parts", lambda: [])():
+                key = part.step_lists_key(block_size) if hasattr(part, "step_lists_key") else None
+                if key is not None and key not in out:
+                    out[key] = part
+        return out
 
     # ------------------------------------------------------------------ cache needs
     def cache_specs(self):
@@ -101,6 +115,10 @@ class Model:
             states.append(None if borrowed else mixer.state_spec())
         return paged, states
 
+    def page_bytes(self, block_size: int) -> int:
+        """Bytes of one page in every cache group of this model (all stops)."""
+        return bytes_of_one_page_everywhere(self.cache_specs()[0], block_size, self.dtype)
+
     def new_cache(self, block_size: int, num_blocks, num_slots: int) -> CacheManager:
         paged, states = self.cache_specs()
         return CacheManager(paged, states, block_size, num_blocks, num_slots, self.dtype, str(self.device))
@@ -112,7 +130,7 @@ class Model:
         self.forward_pass_count += 1
         plan = self.plan
         residual = torch.empty((ctx.num_tokens, plan.hidden_size), dtype=torch.float32, device=self.device)
-        K.embedding(residual, self.embedding, token_ids)
+        K.embedding(residual, self.embedding, token_ids, plan.embedding_scale)
         stream = ResidualStream(residual)
         for index, entry in enumerate(plan.schedule):
             ctx.entry = index
@@ -123,7 +141,10 @@ class Model:
         if rows == 0:
             return torch.empty((0, plan.vocab_size), dtype=torch.float32, device=self.device)
         last = self.final_norm.forward(stream, logit_rows)
-        return self.head.float32(last)
+        logits = self.head.float32(last)
+        if plan.logit_scale != 1.0 or plan.logit_softcap:
+            K.logits_finish(logits, plan.logit_scale, plan.logit_softcap or 0.0)
+        return logits
 
 
 def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") -> Model:
@@ -136,4 +157,20 @@ def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") 
     model.config = config
     weights = load_weights(model_dir, model.expected_tensors(), model.optional_tensors())
     model.bind(weights)
+    return model
+
+
+def random_model(config, seed: int = 0, dtype: str = "bfloat16", device: str = "cuda:0", std: float = 0.02,
+                 norm_std: float = 0.0) -> Model:
+    """A model of `config` (a config.json dict, or a registered architecture's typed config) with
+    random weights drawn on the device, tensor by tensor as the parts bind them: nothing is written
+    to disk and no tensor exists twice, so the 72B shape's 145 GB fit one GPU.  The reference draws
+    random weights only for its tiny test model (tests/tiny_model.py:21-50)."""
+    if dtype not in TORCH_DTYPE:
+        raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
+    if isinstance(config, Mapping):
+        config = read_config_dict(config)
+    model = Model(config.plan(), TORCH_DTYPE[dtype], device)
+    model.config = config
+    model.bind(RandomWeights(model.expected_tensors(), seed, std, norm_std, device))
     return model

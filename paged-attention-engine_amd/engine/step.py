@@ -21,8 +21,7 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..kernels import lib as K
-from ..kernels.lib import PREFILL_TILE  # tokens per run of the prefill attention kernel
-from ..parts import StepContext
+from ..parts import StepContext, StepShape
 from .model import Model
 
 
@@ -42,12 +41,27 @@ class _CapturedStep:
         self.logits: Optional[torch.Tensor] = None
 
 
+def padded_rows(count: int) -> int:
+    """Rows a recorded step of `count` sequences is padded to: every count up to 8, then multiples
+    of 4 up to 32, then multiples of 8.  A stream whose batch shrinks and grows by one sequence
+    at a time then replays a handful of recordings instead of making one per count."""
+    if count <= 8:
+        return count
+    unit = 4 if count <= 32 else 8
+    return -(-count // unit) * unit
+
+
 class StepRunner:
     """Runs steps.  Steps in which every sequence brings exactly one token (decode
     steps) are recorded once per shape as a HIP graph and replayed, so that a step
     costs one copy of its inputs and one graph launch instead of hundreds of kernel
     launches; this needs every part of the model to be `graph_safe` (no host-side
-    data in its forward) and is switched off otherwise."""
+    data in its forward) and is switched off otherwise.
+
+    A recorded step is padded to `padded_rows` sequences.  A padding row is a sequence of its own
+    that holds one token at position 0 in the cache's padding page and padding state slot (which
+    no real sequence ever holds), so it reads and writes nothing that anyone looks at; its
+    logits are dropped."""
 
     TABLE_ROUND = 64    # block tables of captured steps are padded to a multiple of this many pages
     MAX_GRAPHS = 24
@@ -58,8 +72,11 @@ class StepRunner:
         self.device = model.device
         self.vocab_size = model.plan.vocab_size
         self.use_graphs = use_graphs and model.graph_safe
+        self.graph_max_rows = model.graph_max_rows
+        self._list_parts = model.step_list_parts(cache.block_size)
         self._graphs: Dict[tuple, _CapturedStep] = {}
         self.graph_replays = 0
+        self.graph_recordings = 0
 
     def run(self, entries: Sequence[StepEntry],
             feeds: Optional[Tuple[torch.Tensor, Sequence[Tuple[int, int]]]] = None) -> torch.Tensor:
@@ -108,25 +125,37 @@ class StepRunner:
         if not ids:
             raise ValueError("a step needs at least one entry")
 
-        T, S = len(ids), len(seq_ids)
-        decode_only = self.use_graphs and T == S and (self.model.dtype == torch.float32 or S <= 64)
-        decode_tokens = [q_starts[i] for i in range(S) if q_lens[i] == 1]
-        runs = []  # (keys the run sees, tile): runs of at most PREFILL_TILE consecutive tokens of a sequence
-        for i in range(S):
-            if q_lens[i] > 1:
-                for first in range(0, q_lens[i], PREFILL_TILE):
-                    count = min(PREFILL_TILE, q_lens[i] - first)
-                    runs.append((past_lens[i] + first + count, [i, q_starts[i] + first, count]))
-        # the runs with the most keys start first: the last workgroup to finish sets the kernel's time
-        runs.sort(key=lambda run: -run[0])
-        tiles: List[int] = [x for _, tile in runs for x in tile]
-        tables = []
-        for group in cache.groups:
-            per_seq = [cache.block_table(group.index, s) for s in seq_ids]
-            width = max(1, max(len(t) for t in per_seq))
+        T, S, R = len(ids), len(seq_ids), len(rows)
+        per_group = [[cache.table_array(group.index, s) for s in seq_ids] for group in cache.groups]
+        decode_only = (self.use_graphs and T == S
+                       and (self.graph_max_rows is None or padded_rows(S) <= self.graph_max_rows))
+        if decode_only and padded_rows(S) > S:
+            # padding rows: one token each at position 0 of a sequence that lives in the padding page
+            extra = padded_rows(S) - S
+            ids += [ids[0]] * extra
+            positions += [0] * extra
+            tok_seq += list(range(S, S + extra))
+            q_starts += list(range(S, S + extra))
+            q_lens += [1] * extra
+            past_lens += [0] * extra
+            slots += [cache.padding_slot] * extra
+            seq_ids = seq_ids + [-1] * extra
+            per_group = [tables + [array("i", [cache.padding_page(group.index)])] * extra
+                         for group, tables in zip(cache.groups, per_group)]
+            if R == S:  # every sequence samples: the padding rows' logits are computed and dropped
+                rows += list(range(S, S + extra))
+            T = S = S + extra
+        widths = []
+        for tables in per_group:
+            width = max(1, max(len(t) for t in tables))
             if decode_only:
                 width = -(-width // self.TABLE_ROUND) * self.TABLE_ROUND
-            tables.append((width, per_seq))
+            widths.append(width)
+
+        # index lists that parts asked for (their kernels' work lists), built from the step's shape
+        shape = StepShape(tuple(seq_ids), tuple(q_starts), tuple(q_lens), tuple(past_lens), cache.block_size)
+        part_lists = [(key, name, list(flat), width) for key, part in self._list_parts.items()
+                      for name, (flat, width) in part.step_lists(shape).items()]
 
         # one staging buffer, one copy to the device
         # places and rows of token ids that come from the device, padded to one per sequence
@@ -135,24 +164,30 @@ class StepRunner:
             raise ValueError("feeds: at most one per sequence, places within the step, rows within the tokens")
         fed_places = [place for place, _ in fed] + [0] * (S - len(fed))
         fed_rows = [row for _, row in fed] + [0] * (S - len(fed))
-        flat: List[int] = ids + positions + tok_seq + slots + rows + decode_tokens + tiles + fed_places + fed_rows
-        for width, per_seq in tables:
-            for table in per_seq:
+        flat = array("i", ids)
+        for piece in (positions, tok_seq, slots, rows, fed_places, fed_rows):
+            flat.extend(piece)
+        for _, _, values, _ in part_lists:
+            flat.extend(values)
+        for width, tables in zip(widths, per_group):
+            hole = array("i", [-1])
+            for table in tables:
                 flat.extend(table)
-                flat.extend([-1] * (width - len(table)))
-        staging = torch.frombuffer(array("i", flat), dtype=torch.int32).pin_memory()
+                flat.extend(hole * (width - len(table)))
+        staging = torch.frombuffer(flat, dtype=torch.int32).pin_memory()
 
         captured = None
         if decode_only:
-            key = (S, len(rows), tuple(w for w, _ in tables))
-            captured = self._graphs.get(key)
+            key = (S, len(rows), tuple(widths), tuple(len(values) for _, _, values, _ in part_lists))
+            captured = self._graphs.pop(key, None)
             if captured is None:
                 if len(self._graphs) >= self.MAX_GRAPHS:
-                    # the oldest recording goes; a step launched from it may still be running
+                    # the recording that has gone unused the longest goes; a step launched from it
+                    # may still be running
                     torch.cuda.current_stream().synchronize()
                     self._graphs.pop(next(iter(self._graphs)))
-                captured = self._graphs[key] = _CapturedStep(torch.empty(len(flat), dtype=torch.int32,
-                                                                         device=self.device))
+                captured = _CapturedStep(torch.empty(len(flat), dtype=torch.int32, device=self.device))
+            self._graphs[key] = captured  # last used, last to go
             captured.inputs.copy_(staging, non_blocking=True)
             dev = captured.inputs
         else:
@@ -166,19 +201,21 @@ class StepRunner:
             return out
 
         d_ids, d_pos, d_seq, d_slots, d_rows = take(T), take(T), take(T), take(S), take(len(rows))
-        d_decode, d_tiles = take(len(decode_tokens)), take(len(tiles)).view(-1, 3)
         d_fed_places, d_fed_rows = take(S), take(S)
+        memo: Dict[object, object] = {}
+        for key, name, values, width in part_lists:
+            tensor = take(len(values))
+            memo.setdefault(key, {})[name] = tensor.view(-1, width) if width else tensor
         if fed:
             K.scatter_int32(d_ids, d_fed_places, feeds[0], d_fed_rows, len(fed))
         block_tables: Dict[int, torch.Tensor] = {}
-        for group, (width, _) in zip(cache.groups, tables):
+        for group, width in zip(cache.groups, widths):
             block_tables[group.index] = take(S * width).view(S, width)
 
         ctx = StepContext(dtype=self.model.dtype, device=self.device, num_tokens=T, num_seqs=S,
                           positions=d_pos, tok_seq=d_seq, block_tables=block_tables, slots=d_slots,
                           cache=cache, seq_ids=seq_ids, q_starts=q_starts, q_lens=q_lens,
-                          past_lens=past_lens, host_slots=slots, decode_tokens=d_decode,
-                          prefill_tiles=d_tiles)
+                          past_lens=past_lens, host_slots=slots, memo=memo)
         if captured is None:
             return self.model.forward(ctx, d_ids, d_rows)
         if captured.graph is None:
@@ -187,8 +224,9 @@ class StepRunner:
             with torch.cuda.graph(graph):
                 captured.logits = self.model.forward(ctx, d_ids, d_rows)
             captured.graph = graph
+            self.graph_recordings += 1
         else:
             self.model.forward_pass_count += 1
         captured.graph.replay()
         self.graph_replays += 1
-        return captured.logits
+        return captured.logits[:R]

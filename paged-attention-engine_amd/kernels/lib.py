@@ -51,7 +51,8 @@ def _declare(lib) -> None:
     P, I, L, F = c_void_p, c_int, c_int64, c_float
     sig = {
         "pae_device_arch": [c_char_p, I],
-        "pae_embedding": [I, P, P, P, I, I, I, P],
+        "pae_embedding": [I, P, P, P, I, I, I, F, P],
+        "pae_logits_finish": [P, L, F, F, P],
         "pae_add_rmsnorm": [I, P, P, I, L, P, I, F, P, P, I, I, I, P],
         "pae_residual_add": [I, P, P, L, P],
         "pae_scatter_i32": [P, P, P, P, I, P],
@@ -128,14 +129,21 @@ def device_arch() -> str:
     return buf.value.decode().split(":")[0]
 
 
-def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
-    """out[t] = table[ids[t]] as float32; ids int32 (checked against the table by the caller)."""
+def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> None:
+    """out[t] = scale * table[ids[t]] as float32; ids int32 (checked against the table by the caller)."""
     _gpu(out, table, ids)
     T, H = out.shape
     assert out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous()
     assert ids.dtype == torch.int32 and ids.numel() == T and table.shape[1] == H
     _check(library().pae_embedding(code_of(table.dtype), out.data_ptr(), table.data_ptr(), ids.data_ptr(),
-                                   T, H, table.shape[0], _stream()))
+                                   T, H, table.shape[0], float(scale), _stream()))
+
+
+def logits_finish(logits: torch.Tensor, scale: float = 1.0, softcap: float = 0.0) -> None:
+    """In place: logits = scale * logits, then with a soft cap c > 0, c * tanh(logits / c)."""
+    _gpu(logits)
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    _check(library().pae_logits_finish(logits.data_ptr(), logits.numel(), float(scale), float(softcap), _stream()))
 
 
 def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
@@ -227,6 +235,18 @@ def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, cos_s
                                        _ptr(cos_sin) if rot else None, positions.data_ptr(), _ptr(tok_seq),
                                        _ptr(block_tables), max_blocks, block_size, _ptr(k_cache), _ptr(v_cache),
                                        1 if write else 0, _stream()))
+
+
+def rotate_heads(x: torch.Tensor, num_heads: int, hd: int, rot: int, cos_sin: torch.Tensor,
+                 positions: torch.Tensor) -> None:
+    """Rotate the first `num_heads` heads (each `hd` wide) of every row of `x` in place; nothing is stored."""
+    rope_kv_write(x, num_heads, 0, hd, rot, cos_sin, positions, None, None, 1, None, None)
+
+
+def kv_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, positions: torch.Tensor, tok_seq: torch.Tensor,
+             block_tables: torch.Tensor, block_size: int, k_cache: torch.Tensor, v_cache: torch.Tensor) -> None:
+    """Copy the key and value heads of rows [q heads | k heads | v heads] into their cache slots, as they are."""
+    rope_kv_write(qkv, nh, nkv, hd, 0, None, positions, tok_seq, block_tables, block_size, k_cache, v_cache)
 
 
 def swiglu(out: torch.Tensor, x: torch.Tensor, block: int = 0) -> None:

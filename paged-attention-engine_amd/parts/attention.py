@@ -8,6 +8,12 @@ up to its own position (engine/attention.py:474-487), heads merged, output
 projection.  The three projections are one product over concatenated weights;
 row-wise dot products are unchanged by the concatenation.
 
+The mixer owns its cache: it declares the pages it keeps (`paged_spec`), stores new
+keys and values itself, and builds the work lists of its kernels from the step's shape
+(`step_lists`).  The position encoding only encodes; when it is a rotation that hands
+out its table, the rotation runs inside the mixer's fused kernels (projection +
+rotation + store for up to 64 rows, rotation + store above).
+
 A stop that borrows another stop's cache projects queries only and reads keys
 and values written by the owner.
 """
@@ -16,17 +22,32 @@ from __future__ import annotations
 
 import torch
 
-from ..cache.manager import PagedSpec
+from ..cache.manager import attention_pages
 from ..kernels import lib as K
-from .base import POSITION_ENCODINGS, Part, build_part, register_mixer
-from .linear import Linear
+from .base import POSITION_ENCODINGS, Part, StepShape, build_part, register_mixer
+from .linear import Linear, rows_a_graph_may_hold
+
+WORK_LISTS = ("paged attention work lists", K.PREFILL_TILE)
+
+
+def attention_work_lists(shape: StepShape):
+    """What the matrix-core attention kernels walk: `decode_tokens`, the flat rows of sequences that
+    bring one token, and `prefill_tiles`, runs of up to PREFILL_TILE consecutive tokens of the
+    others as (table row, first flat token, count).  The runs with the most keys come first:
+    workgroups start in list order, and the last to finish sets the kernel's time."""
+    decode_tokens = [start for start, n in zip(shape.q_starts, shape.q_lens) if n == 1]
+    runs = []
+    for row, (start, n, past) in enumerate(zip(shape.q_starts, shape.q_lens, shape.past_lens)):
+        if n > 1:
+            for first in range(0, n, K.PREFILL_TILE):
+                count = min(K.PREFILL_TILE, n - first)
+                runs.append((past + first + count, (row, start + first, count)))
+    runs.sort(key=lambda run: -run[0])
+    return {"decode_tokens": (decode_tokens, 0), "prefill_tiles": ([x for _, tile in runs for x in tile], 3)}
 
 
 @register_mixer("attention")
 class PagedAttention(Part):
-    @property
-    def graph_safe(self) -> bool:
-        return self.position.graph_safe
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         if spec.num_heads % spec.num_kv_heads:
@@ -37,11 +58,26 @@ class PagedAttention(Part):
                          if spec.position is not None else
                          POSITION_ENCODINGS["none"](None, dtype, device))
 
-    def product_widths(self):
-        return [self.spec.hidden_size, self.spec.num_heads * self.spec.head_dim]
+    @property
+    def graph_safe(self) -> bool:
+        return self.position.graph_safe
+
+    @property
+    def graph_max_rows(self):
+        return rows_a_graph_may_hold(self.dtype, self.spec.hidden_size, self.spec.num_heads * self.spec.head_dim)
 
     def paged_spec(self):
-        return PagedSpec(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)
+        return attention_pages(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)
+
+    def _matrix_cores(self, block_size: int) -> bool:
+        s = self.spec
+        return K.mfma_attention_supported(self.dtype, s.num_heads, s.num_kv_heads, s.head_dim, block_size)
+
+    def step_lists_key(self, block_size: int):
+        return WORK_LISTS if self._matrix_cores(block_size) else None
+
+    def step_lists(self, shape: StepShape):
+        return attention_work_lists(shape)
 
     def tensors(self, prefix):
         s = self.spec
@@ -68,34 +104,51 @@ class PagedAttention(Part):
         ob = weights.get(prefix + "o_proj.bias") if s.out_bias else None
         self.out = Linear(self.matrix(weights[prefix + "o_proj.weight"]), None if ob is None else self.vector(ob))
 
+    def _project_encode_store(self, ctx, x, k_cache, v_cache, table):
+        """Queries (and, at a stop that owns its cache, keys and values) of the step's tokens:
+        projected, encoded by position, the new keys and values stored.  Returns rows whose first
+        num_heads * head_dim features are the encoded queries."""
+        s = self.spec
+        bs = ctx.cache.block_size
+        if ctx.writes_cache:
+            linear, nkv = self.qkv, s.num_kv_heads
+        else:
+            linear, nkv, k_cache, v_cache, table = self.q_only, 0, None, None, None
+        rotary = getattr(self.position, "rotary_table", None)
+        if rotary is None:
+            # any encoding: project, let it encode query and key heads in place, then store
+            qkv = linear(x)
+            self.position.encode(ctx, qkv, s.num_heads + nkv, s.head_dim)
+            if nkv:
+                K.kv_store(qkv, s.num_heads, nkv, s.head_dim, ctx.positions, ctx.tok_seq, table, bs, k_cache, v_cache)
+            return qkv
+        rot, cos_sin = rotary(ctx)
+        if x.dtype == torch.bfloat16 and K.skinny_rope_supported(x, linear.weight, s.head_dim, rot):
+            # up to 64 rows: one kernel projects, rotates and stores
+            q = torch.empty((x.shape[0], s.num_heads * s.head_dim), dtype=x.dtype, device=x.device)
+            splits = K.whole_sum_splits(linear.out_features, linear.in_features, x.shape[0])
+            K.gemm_skinny_rope(q, x, linear.weight, linear.bias, s.num_heads, nkv, s.head_dim, rot, cos_sin,
+                               ctx.positions, ctx.tok_seq, table, bs, k_cache, v_cache, splits)
+            return q
+        qkv = linear(x)
+        K.rope_kv_write(qkv, s.num_heads, nkv, s.head_dim, rot, cos_sin, ctx.positions, ctx.tok_seq, table, bs,
+                        k_cache, v_cache)
+        return qkv
+
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         s = self.spec
-        group = ctx.cache.group_of(ctx.cache_entry)
         k_cache, v_cache = ctx.cache.kv_of(ctx.cache_entry)
-        table = ctx.block_tables[group]
-        # a position encoding may offer the projection, its encoding and the cache write as one step
-        fused = getattr(self.position, "project_encode_store", None)
-        if ctx.writes_cache:
-            stored = (s.num_kv_heads, s.head_dim, k_cache, v_cache, table, ctx.cache.block_size)
-            qkv = fused(ctx, x, self.qkv, s.num_heads, *stored) if fused else None
-            if qkv is None:
-                qkv = self.qkv(x)
-                self.position.encode_and_store(ctx, qkv, s.num_heads, *stored)
-        else:
-            stored = (0, s.head_dim, None, None, None, ctx.cache.block_size)
-            qkv = fused(ctx, x, self.q_only, s.num_heads, *stored) if fused else None
-            if qkv is None:
-                qkv = self.q_only(x)
-                self.position.encode_and_store(ctx, qkv, s.num_heads, *stored)
+        table = ctx.block_tables[ctx.cache.group_of(ctx.cache_entry)]
+        qkv = self._project_encode_store(ctx, x, k_cache, v_cache, table)
         attn = torch.empty((x.shape[0], s.num_heads * s.head_dim), dtype=x.dtype, device=x.device)
         geometry = (s.num_heads, s.num_kv_heads, s.head_dim, s.scale, s.window or 0)
-        if K.mfma_attention_supported(x.dtype, s.num_heads, s.num_kv_heads, s.head_dim, ctx.cache.block_size) \
-                and ctx.decode_tokens is not None:
-            if ctx.decode_tokens.numel():
-                K.attn_decode(attn, qkv, k_cache, v_cache, ctx.decode_tokens, ctx.positions, ctx.tok_seq, table,
-                              *geometry)
-            if ctx.prefill_tiles.numel():
-                K.attn_prefill(attn, qkv, k_cache, v_cache, ctx.prefill_tiles, ctx.positions, table, *geometry)
+        work = ctx.memo.get(WORK_LISTS) if self._matrix_cores(ctx.cache.block_size) else None
+        if work is not None:
+            decode_tokens, prefill_tiles = work["decode_tokens"], work["prefill_tiles"]
+            if decode_tokens.numel():
+                K.attn_decode(attn, qkv, k_cache, v_cache, decode_tokens, ctx.positions, ctx.tok_seq, table, *geometry)
+            if prefill_tiles.numel():
+                K.attn_prefill(attn, qkv, k_cache, v_cache, prefill_tiles, ctx.positions, table, *geometry)
         else:
             K.paged_attention_generic(attn, qkv, k_cache, v_cache, ctx.positions, ctx.tok_seq, table, *geometry)
         return self.out.branch(attn)

@@ -4,8 +4,8 @@ A model is put together from five kinds of parts, each chosen by the `kind` of
 its spec and none aware of the model it sits in:
 
   norm               forward(stream, rows=None) -> normalised activations
-  position encoding  encode_and_store(ctx, qkv, ...): rotates queries/keys, writes the cache
-  mixer              forward(ctx, x) -> y        (attention here; may keep paged or per-request state)
+  position encoding  encode(ctx, x, num_heads, head_dim): encodes heads in place by the tokens' positions
+  mixer              forward(ctx, x) -> y        (attention here; keeps what it caches, paged or per request)
   feed-forward       forward(ctx, x) -> y
   block              forward(ctx, stream)        (arranges two norms, a mixer and a feed-forward)
 
@@ -35,6 +35,23 @@ class ResidualStream:
         self.pending: Optional[torch.Tensor] = None
 
 
+@dataclass(frozen=True)
+class StepShape:
+    """A step on the host, before anything is on the device: which sequences bring how many
+    tokens at which place.  Parts that want index lists of their own for a step (work lists of
+    a kernel, say) build them from this; see `Part.step_lists`."""
+
+    seq_ids: Tuple[int, ...]
+    q_starts: Tuple[int, ...]   # first flat row of each sequence
+    q_lens: Tuple[int, ...]     # rows of each sequence in this step
+    past_lens: Tuple[int, ...]  # tokens each sequence held before the step
+    block_size: int
+
+    @property
+    def num_tokens(self) -> int:
+        return sum(self.q_lens)
+
+
 @dataclass
 class StepContext:
     """One step as parts see it: flat tokens of several sequences and their caches."""
@@ -54,16 +71,13 @@ class StepContext:
     q_lens: List[int] = field(default_factory=list)     # rows of each sequence in this step
     past_lens: List[int] = field(default_factory=list)  # tokens each sequence held before the step
     host_slots: List[int] = field(default_factory=list)
-    # work lists of the attention kernels: sequences that bring one token, and runs of up to 64
-    # consecutive tokens of the others as (table row, first flat token, count), most keys first
-    decode_tokens: Optional[torch.Tensor] = None   # int32 [number of single-token sequences]
-    prefill_tiles: Optional[torch.Tensor] = None   # int32 [runs of 2..64 tokens, 3]: table row, first token, count
     # set by the model for the stop that is running
     entry: int = 0                     # index in the schedule
     cache_entry: int = 0               # the stop whose cache is read (entry itself unless it borrows)
     writes_cache: bool = True
     # what a part computes once per step for every layer that has the same part (a table of angles,
-    # say), under a key of the part's choosing
+    # say), under a key of the part's choosing; the step function also leaves here, under
+    # `step_lists_key`, the index lists a part asked for (`Part.step_lists`), as int32 device tensors
     memo: Dict[object, object] = field(default_factory=dict)
 
 
@@ -74,6 +88,9 @@ class Part:
     # data (nothing read from the context's host lists, no synchronisation): such a
     # part can be recorded into a HIP graph and replayed with new inputs.
     graph_safe = False
+    # The most rows of a step for which that holds (None: any number): a part whose products
+    # leave this engine's kernels above some row count says so here.
+    graph_max_rows: Optional[int] = None
 
     def __init__(self, spec, dtype: torch.dtype, device) -> None:
         self.spec = spec
@@ -95,6 +112,17 @@ class Part:
         """A norm weight or bias: stays float32 if stored so, else the compute precision."""
         keep = torch.float32 if t.dtype == torch.float32 else self.dtype
         return t.to(device=self.device, dtype=keep).contiguous()
+
+    # Index lists of the part's own for every step (a kernel's work lists, for instance).  A part
+    # that wants them names a key (parts with equal keys share one set of lists per step) and
+    # builds them on the host from the step's shape: {name: (flat list of ints, row width or 0)}.
+    # The step function copies them to the device with its own metadata, in the same transfer,
+    # and leaves {name: int32 tensor} in `ctx.memo[key]` (viewed [-1, width] when a width is given).
+    def step_lists_key(self, block_size: int):
+        return None
+
+    def step_lists(self, shape: "StepShape"):
+        return {}
 
     # what the part keeps in the cache (mixers override)
     def paged_spec(self):

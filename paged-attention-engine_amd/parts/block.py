@@ -23,12 +23,14 @@ class PreNormBlock:
     def graph_safe(self) -> bool:
         return all(part.graph_safe for part, _ in self._named())
 
-    def product_widths(self):
-        """Inner dimensions of the block's matrix products (the skinny kernel wants multiples of 8)."""
-        out = []
-        for part, _ in self._named():
-            out += getattr(part, "product_widths", lambda: [])()
-        return out
+    @property
+    def graph_max_rows(self):
+        """The fewest rows any part allows a recorded step to hold (None: no part sets a limit)."""
+        limits = [part.graph_max_rows for part, _ in self._named() if part.graph_max_rows is not None]
+        return min(limits) if limits else None
+
+    def parts(self):
+        return [part for part, _ in self._named()]
 
     def _named(self):
         s = self.spec

@@ -21,12 +21,25 @@ import torch
 from ..kernels import lib as K
 
 
+def rows_a_graph_may_hold(dtype: torch.dtype, *inner_sizes: int):
+    """For products with these inner sizes: up to how many rows every one of them runs in this
+    engine's own kernels, which is what recording a step as a HIP graph needs (library products
+    may record memory clears into a graph).  None: any number of rows; 0: never."""
+    if dtype == torch.float32:
+        return None
+    return K.SKINNY_MAX_ROWS if all(size % 8 == 0 for size in inner_sizes) else 0
+
+
 class Linear:
     def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:
         assert weight.dim() == 2 and weight.is_contiguous()
         self.weight = weight
         self.bias = bias
         self.out_features, self.in_features = weight.shape
+
+    @property
+    def graph_max_rows(self):
+        return rows_a_graph_may_hold(self.weight.dtype, self.in_features)
 
     def _library(self, x: torch.Tensor) -> torch.Tensor:
         out = torch.empty((x.shape[0], self.out_features), dtype=x.dtype, device=x.device)

@@ -8,7 +8,7 @@ import torch
 
 from ..kernels import lib as K
 from .base import Part, register_feed_forward
-from .linear import Linear
+from .linear import Linear, rows_a_graph_may_hold
 
 
 @register_feed_forward("swiglu")
@@ -19,8 +19,9 @@ class SwiGLU(Part):
         if spec.activation != "silu":
             raise ValueError(f"activation '{spec.activation}' is not supported by the gated feed-forward")
 
-    def product_widths(self):
-        return [self.spec.hidden_size, self.spec.intermediate_size]
+    @property
+    def graph_max_rows(self):
+        return rows_a_graph_may_hold(self.dtype, self.spec.hidden_size, self.spec.intermediate_size)
 
     def tensors(self, prefix):
         s = self.spec

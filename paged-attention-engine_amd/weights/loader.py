@@ -42,12 +42,25 @@ def _open_shards(model_dir: str) -> Dict[str, SafetensorsFile]:
     files: Dict[str, SafetensorsFile] = {}
     by_name: Dict[str, SafetensorsFile] = {}
     if os.path.exists(index_path):
-        with open(index_path, "r", encoding="utf-8") as handle:
-            weight_map = json.load(handle)["weight_map"]
+        try:
+            with open(index_path, "r", encoding="utf-8") as handle:
+                weight_map = json.load(handle)["weight_map"]
+        except (json.JSONDecodeError, KeyError, TypeError) as err:
+            raise WeightsError(f"{index_path}: not a shard index with a 'weight_map' ({err})") from err
+        absent = []  # names the index sends to a shard that does not hold them
         for name, shard in weight_map.items():
             if shard not in files:
-                files[shard] = SafetensorsFile(os.path.join(model_dir, shard))
-            by_name[name] = files[shard]
+                shard_path = os.path.join(model_dir, shard)
+                if not os.path.exists(shard_path):
+                    raise WeightsError(f"{index_path} names the shard {shard}, which is not in the folder")
+                files[shard] = SafetensorsFile(shard_path)
+            if name in files[shard].entries:
+                by_name[name] = files[shard]
+            else:
+                absent.append(f"{name} (not in {shard})")
+        if absent:
+            raise WeightsError(f"{index_path}: the index names tensors that their shards lack: "
+                               + ", ".join(sorted(absent)), missing=[a.split(" ")[0] for a in absent])
     elif os.path.exists(single):
         shard = SafetensorsFile(single)
         for name in shard.names():
@@ -65,13 +78,35 @@ def _keep_precision(t: torch.Tensor) -> torch.Tensor:
     return t.to(torch.int32)
 
 
+class FolderWeights(Mapping):
+    """name -> tensor of a checked folder.  A lookup returns a view of the memory-mapped file (a
+    converting copy only for precisions that are not kept), so a part that sends it to the device
+    copies straight from the file's pages: no second copy of the model ever sits in host memory.
+    The views are private to this process (copy-on-write); the files stay open while the mapping
+    lives."""
+
+    def __init__(self, by_name: Mapping[str, SafetensorsFile], names) -> None:
+        self._by_name = {name: by_name[name] for name in names}
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        return _keep_precision(self._by_name[name].tensor(name))
+
+    def __iter__(self):
+        return iter(self._by_name)
+
+    def __len__(self) -> int:
+        return len(self._by_name)
+
+
 def load_weights(model_dir: str, expected: Mapping[str, Tuple[int, ...]],
-                 optional: Sequence[str] = (), device: Optional[str] = None) -> Dict[str, torch.Tensor]:
+                 optional: Sequence[str] = (), device: Optional[str] = None) -> Mapping[str, torch.Tensor]:
     """Tensors named in `expected`, each with exactly the declared shape.
 
     `optional` names may be present in the folder without being expected (a tied
     head that a file stores anyway); they are ignored.  Anything else that the
-    folder holds and the model does not declare is reported as unexpected."""
+    folder holds and the model does not declare is reported as unexpected.
+    Without `device` the result is a `FolderWeights` over the mapped files; with
+    one, a dict of tensors on that device."""
     try:
         by_name = _open_shards(model_dir)
     except SafetensorsError as err:
@@ -90,8 +125,7 @@ def load_weights(model_dir: str, expected: Mapping[str, Tuple[int, ...]],
             lines.append(f"  wrong shape ({len(wrong)}): " + "; ".join(
                 f"{n} is {list(got)}, model needs {list(want)}" for n, got, want in sorted(wrong)))
         raise WeightsError("\n".join(lines), missing, unexpected, wrong)
-    out = {}
-    for name in expected:
-        t = _keep_precision(by_name[name].tensor(name))
-        out[name] = t.to(device) if device is not None else t.clone()
-    return out
+    weights = FolderWeights(by_name, expected)
+    if device is None:
+        return weights
+    return {name: weights[name].to(device) for name in expected}

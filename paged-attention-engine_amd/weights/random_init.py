@@ -8,7 +8,11 @@ as bfloat16, the precision checkpoints of this family ship in, so that the
 32-bit and the bfloat16 paths start from the same numbers.
 
 Every tensor has a generator of its own, seeded from (seed, name): any tensor
-can be produced alone, on the CPU or on the device that will hold it.
+can be produced alone, on the CPU or on the device that will hold it (the two
+devices' generators give different numbers for one seed; a folder is always drawn
+on the CPU).  `RandomWeights` is the mode for models too large to write out: a
+read-only mapping that draws each tensor on the device at the moment a part asks
+for it and keeps none, so that 145 GB of weights never exist twice.
 """
 
 from __future__ import annotations
@@ -16,7 +20,7 @@ from __future__ import annotations
 import json
 import os
 import zlib
-from typing import Dict, Mapping, Tuple
+from typing import Dict, Iterator, Mapping, Tuple
 
 import torch
 
@@ -50,6 +54,28 @@ def random_weights(expected: Mapping[str, Tuple[int, ...]], seed: int, std: floa
                    dtype: torch.dtype = torch.bfloat16) -> Dict[str, torch.Tensor]:
     return {name: random_tensor(name, tuple(shape), seed, std, norm_std, device, dtype)
             for name, shape in expected.items()}
+
+
+class RandomWeights(Mapping):
+    """name -> tensor, drawn anew at every lookup on `device` from (seed, name); nothing is kept.
+    Two lookups of one name give equal tensors, so the same mapping can feed a model and, in a
+    test, the plain implementation it is compared with."""
+
+    def __init__(self, expected: Mapping[str, Tuple[int, ...]], seed: int, std: float = 0.02,
+                 norm_std: float = 0.0, device: str = "cuda:0", dtype: torch.dtype = torch.bfloat16) -> None:
+        self.shapes = {name: tuple(shape) for name, shape in expected.items()}
+        self.seed, self.std, self.norm_std, self.device, self.dtype = seed, std, norm_std, device, dtype
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        if name not in self.shapes:
+            raise KeyError(name)
+        return random_tensor(name, self.shapes[name], self.seed, self.std, self.norm_std, self.device, self.dtype)
+
+    def __iter__(self) -> Iterator[str]:
+        return iter(self.shapes)
+
+    def __len__(self) -> int:
+        return len(self.shapes)
 
 
 def write_model_folder(config, seed: int, out_dir: str, std: float = 0.02, norm_std: float = 0.0,

@@ -6,7 +6,7 @@ import random
 
 import pytest
 
-from paged_attention_engine_amd.cache import (HOLE, AllocStatus, BlockAllocator, CacheManager, PagedSpec,
+from paged_attention_engine_amd.cache import (HOLE, AllocStatus, BlockAllocator, CacheManager, PagedSpec, attention_pages,
                                               StateSpec)
 
 
@@ -114,7 +114,7 @@ def test_window_pages_come_back_and_leave_holes():
 
 
 def two_group_manager(num_blocks=6, slots=3):
-    paged = [PagedSpec(2, 16), PagedSpec(2, 16), PagedSpec(2, 16, window=6), PagedSpec(2, 16, window=6), None]
+    paged = [attention_pages(2, 16), attention_pages(2, 16), attention_pages(2, 16, window=6), attention_pages(2, 16, window=6), None]
     states = [None, None, None, None, StateSpec((4,))]
     return CacheManager(paged, states, block_size=4, num_blocks=num_blocks, num_slots=slots, device=None)
 

@@ -1,7 +1,9 @@
 """Each part alone against the plain functions, and the framework's generality: a toy
-mixer with state of its own, a toy position encoding and a toy architecture whose schedule
-names a layer twice and lets a stop read another stop's cache are registered here, built
-and stepped (in portions, several sequences at once) without touching the framework's files."""
+mixer with state of its own, a toy mixer that caches one tensor of its own shape per token, a toy
+position encoding (which only encodes: it never sees a cache) and a toy architecture whose
+schedule names a layer twice, lets a stop read another stop's cache and scales its embedding and
+its logits are registered here, built and stepped (in portions, several sequences at once)
+without touching the framework's files."""
 
 import math
 
@@ -10,7 +12,8 @@ import torch
 
 import paged_attention_engine_amd as pae
 from paged_attention_engine_amd import parts as P
-from paged_attention_engine_amd.cache import CacheManager, PagedSpec, StateSpec
+from paged_attention_engine_amd.cache import PAGE, CacheManager, PagedSpec, PagedTensor, StateSpec
+from paged_attention_engine_amd.parts.attention import WORK_LISTS, attention_work_lists
 from paged_attention_engine_amd.config import (FeedForwardSpec, LayerSpec, MixerSpec, ModelPlan, NormSpec, PartSpec,
                                                PositionSpec, ScheduleEntry)
 from tests.plain import qwen2_plain as plain
@@ -36,16 +39,16 @@ def make_ctx(cache, dtype, seq_ids, q_lens):
         width = max(len(r) for r in rows)
         tables[group.index] = torch.tensor([list(r) + [-1] * (width - len(r)) for r in rows], dtype=torch.int32, device=DEV)
     slots = [cache.slot_of(s) for s in seq_ids]
-    dec = [q_starts[i] for i, n in enumerate(q_lens) if n == 1]
-    tiles = [[i, q_starts[i] + f, min(64, n - f)] for i, n in enumerate(q_lens) if n > 1 for f in range(0, n, 64)]
+    # the attention kernels' work lists, as the step function would leave them for the mixer
+    shape = P.StepShape(tuple(seq_ids), tuple(q_starts), tuple(q_lens), tuple(past), cache.block_size)
+    lists = {name: torch.tensor(flat, dtype=torch.int32, device=DEV).view(*((-1, width) if width else (-1,)))
+             for name, (flat, width) in attention_work_lists(shape).items()}
     return P.StepContext(
         dtype=dtype, device=torch.device(DEV), num_tokens=len(positions), num_seqs=len(seq_ids),
         positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
         tok_seq=torch.tensor(tok_seq, dtype=torch.int32, device=DEV), block_tables=tables,
         slots=torch.tensor(slots, dtype=torch.int32, device=DEV), cache=cache, seq_ids=list(seq_ids),
-        q_starts=q_starts, q_lens=list(q_lens), past_lens=past, host_slots=slots,
-        decode_tokens=torch.tensor(dec, dtype=torch.int32, device=DEV),
-        prefill_tiles=torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 3))
+        q_starts=q_starts, q_lens=list(q_lens), past_lens=past, host_slots=slots, memo={WORK_LISTS: lists})
 
 
 # ------------------------------------------------------------------ built-in parts, one at a time
@@ -153,16 +156,12 @@ class DecayMixer(P.Part):
 
 @P.register_position_encoding("toy_shift")
 class ShiftEncoding(P.Part):
-    """Adds position / 100 to the first feature of every query and key head (a toy)."""
+    """Adds position / 100 to the first feature of every head it is given (a toy).  It encodes in
+    place and knows of no cache: the mixer stores keys and values."""
 
-    def encode_and_store(self, ctx, qkv, nh, nkv, hd, k_cache, v_cache, block_table, block_size):
-        from paged_attention_engine_amd.kernels import lib as K
-        heads = qkv.view(qkv.shape[0], -1, hd)
-        rotated = nh + (nkv if k_cache is not None else 0)
-        heads[:, :rotated, 0] += (ctx.positions.float() / 100.0).to(qkv.dtype)[:, None]
-        if k_cache is not None:
-            K.rope_kv_write(qkv, nh, nkv, hd, 0, None, ctx.positions, ctx.tok_seq, block_table, block_size,
-                            k_cache, v_cache)
+    def encode(self, ctx, x, num_heads, head_dim):
+        heads = x[:, :num_heads * head_dim].view(x.shape[0], num_heads, head_dim)
+        heads[:, :, 0] += (ctx.positions.float() / 100.0).to(x.dtype)[:, None]
 
 
 from dataclasses import dataclass
@@ -232,17 +231,18 @@ class ToyConfig:
         ffn = FeedForwardSpec(hidden_size=H, intermediate_size=c["inter"])
         layers = (LayerSpec("layers.0.", attn, ffn, norm, norm), LayerSpec("layers.1.", DecaySpec(hidden_size=H, decay=c["decay"]), ffn, norm, norm))
         schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(0, cache_from=0), ScheduleEntry(1))
-        return ModelPlan("ToyForCausalLM", H, c["vocab"], layers, schedule, norm, "embed.weight", "head.weight", "final_norm.")
+        return ModelPlan("ToyForCausalLM", H, c["vocab"], layers, schedule, norm, "embed.weight", "head.weight", "final_norm.",
+                         embedding_scale=c["embedding_scale"], logit_scale=c["logit_scale"], logit_softcap=c["logit_softcap"])
 
 
 pae.register_architecture("ToyForCausalLM", ToyConfig)
 TOY = dict(architectures=["ToyForCausalLM"], hidden_size=48, head_dim=16, heads=3, kv_heads=1, inter=64, vocab=97,
-           eps=1e-5, decay=0.6)
+           eps=1e-5, decay=0.6, embedding_scale=3.0, logit_scale=0.25, logit_softcap=2.0)
 
 
 def toy_plain_logits(w, c, ids):
     """The toy architecture written out plainly (float64, whole sequence, no cache)."""
-    x = w["embed.weight"][ids].double()
+    x = c["embedding_scale"] * w["embed.weight"][ids].double()
     n = len(ids)
     pos = torch.arange(n, dtype=torch.float64)
     kv_of_stop0 = None
@@ -280,7 +280,9 @@ def toy_plain_logits(w, c, ids):
         x = x + y
         h = plain.rms_norm(x, w[p + "post_attention_layernorm.weight"].double(), c["eps"])
         x = x + plain.swiglu_mlp({k: v.double() for k, v in w.items()}, p, h)
-    return plain.linear(plain.rms_norm(x, w["final_norm.weight"].double(), c["eps"]), w["head.weight"].double())
+    logits = c["logit_scale"] * plain.linear(plain.rms_norm(x, w["final_norm.weight"].double(), c["eps"]),
+                                             w["head.weight"].double())
+    return c["logit_softcap"] * torch.tanh(logits / c["logit_softcap"])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -360,3 +362,84 @@ def helpers_tol(dtype, top):
     from tests import helpers
     ref = torch.tensor(top)
     return helpers.fp32_atol(ref) * 4 if dtype == "float32" else helpers.bf16_atol(ref)
+
+
+# ------------------------------------------------------------------ a mixer with a cached tensor of its own
+@dataclass(frozen=True)
+class LatentSpec(PartSpec):
+    hidden_size: int = 0
+    latent_size: int = 0
+    window: int = 0
+    kind: str = "toy_latent"
+
+
+@P.register_mixer("toy_latent")
+class LatentMeanMixer(P.Part):
+    """Caches one latent vector per token, l_t = W_in x_t, in pages of its own shape [PAGE][latent]
+    (no keys, no values, no heads), and returns W_out applied to the mean of the latents of the last
+    `window` tokens.  Host loops and library calls: a test part."""
+
+    def paged_spec(self):
+        return PagedSpec((PagedTensor("latent", (PAGE, self.spec.latent_size)),), self.spec.window)
+
+    def tensors(self, prefix):
+        s = self.spec
+        return {prefix + "in.weight": (s.latent_size, s.hidden_size), prefix + "out.weight": (s.hidden_size, s.latent_size)}
+
+    def bind(self, prefix, weights):
+        self.w_in = weights[prefix + "in.weight"].to(device=self.device, dtype=torch.float32)
+        self.w_out = weights[prefix + "out.weight"].to(device=self.device, dtype=torch.float32)
+
+    def forward(self, ctx, x):
+        pages = ctx.cache.pages_of(ctx.cache_entry)["latent"]  # [block][page][latent]
+        tables = ctx.block_tables[ctx.cache.group_of(ctx.cache_entry)].cpu()
+        bs, window = ctx.cache.block_size, self.spec.window
+        latents = x.float() @ self.w_in.t()
+        out = torch.empty((x.shape[0], self.spec.hidden_size), dtype=torch.float32, device=x.device)
+        for row, (start, n, past) in enumerate(zip(ctx.q_starts, ctx.q_lens, ctx.past_lens)):
+            for i in range(n):  # store first: a token sees itself
+                pos = past + i
+                pages[int(tables[row, pos // bs]), pos % bs] = latents[start + i].to(pages.dtype)
+            for i in range(n):
+                pos = past + i
+                seen = [pages[int(tables[row, p // bs]), p % bs].float() for p in range(max(0, pos - window + 1), pos + 1)]
+                out[start + i] = torch.stack(seen).mean(0) @ self.w_out.t()
+        return out.to(x.dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_mixer_with_one_cached_tensor_per_token(dtype):
+    """The cache manager builds the pool a mixer declares, whatever its tensors are called and
+    shaped; a window gives pages back, and they are used again by the next request."""
+    torch.manual_seed(4)
+    H, L, window, bs = 40, 24, 10, 4
+    spec = LatentSpec(hidden_size=H, latent_size=L, window=window)
+    part = P.build_part(P.MIXERS, "mixer", spec, DT[dtype], DEV)
+    w = {n: (torch.randn(shape) * 0.3) for n, shape in part.tensors("m.").items()}
+    part.bind("m.", w)
+    cache = CacheManager([part.paged_spec()], [None], bs, 6, 2, DT[dtype], DEV)
+    assert set(cache.groups[0].pools) == {"latent"}
+    assert tuple(cache.groups[0].pools["latent"].shape) == (1, 6 + 1, bs, L)
+    assert cache.storage_bytes() == 6 * bs * L * torch.empty((), dtype=DT[dtype]).element_size()
+
+    def expected(x):
+        lat = (x.float() @ w["m.in.weight"].t()).to(DT[dtype]).float()  # as stored
+        rows = [lat[max(0, t - window + 1):t + 1].mean(0) @ w["m.out.weight"].t() for t in range(x.shape[0])]
+        return torch.stack(rows)
+
+    used = set()
+    for seq, portions in ((0, (7, 1, 9, 2, 6, 8)), (1, (20, 1, 1))):  # 33 tokens need 9 pages without the window
+        x = torch.randn(sum(portions), H).to(DT[dtype])
+        want = expected(x)
+        assert cache.create_sequence(seq)
+        done = 0
+        for n in portions:
+            assert cache.reserve(seq, n).ok
+            used |= {b for b in cache.block_table(0, seq) if b >= 0}
+            ctx = make_ctx(cache, DT[dtype], [seq], [n])
+            got = part.forward(ctx, x[done:done + n].to(DEV))
+            assert (got.float().cpu() - want[done:done + n]).abs().max() <= TOL[dtype] * max(1.0, float(want.abs().max()))
+            done += n
+            cache.release_passed(seq)
+        cache.free_sequence(seq)
+    assert cache.free_blocks() == (6,) and used == set(range(6))

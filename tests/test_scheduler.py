@@ -9,7 +9,7 @@ is a scheduling fault.  The fixtures are the reference's, as behaviours.
 import pytest
 
 from paged_attention_engine_amd import CacheManager, EventKind, Request, Scheduler
-from paged_attention_engine_amd.cache import PagedSpec, StateSpec
+from paged_attention_engine_amd.cache import PagedSpec, attention_pages, StateSpec
 
 VOCAB = 64
 
@@ -34,7 +34,7 @@ class StubExecutor:
 
 
 def make(num_blocks, block_size=4, window=None, slots=64, **kw):
-    cache = CacheManager([PagedSpec(1, 1, window)], [None], block_size, num_blocks, slots, device=None)
+    cache = CacheManager([attention_pages(1, 1, window)], [None], block_size, num_blocks, slots, device=None)
     executor = StubExecutor(cache)
     return Scheduler(executor, cache, **kw), cache, executor
 
@@ -349,7 +349,7 @@ def test_overlapped_steps_decide_and_generate_what_single_steps_do(seed):
     kw = dict(max_num_seqs=rng.choice([None, 2, 4]), max_num_batched_tokens=rng.choice([None, 7, 16]))
 
     def run(overlapped):
-        cache = CacheManager([PagedSpec(1, 1, None)], [None], 4, num_blocks, 64, device=None)
+        cache = CacheManager([attention_pages(1, 1, None)], [None], 4, num_blocks, 64, device=None)
         executor = LaunchingExecutor(cache)
         sched = Scheduler(executor, cache, **kw)
         for r in reqs:
