@@ -3,16 +3,19 @@
 //
 // W is stored (out_features, in_features) row-major as in the checkpoint, the
 // layout F.linear takes in the reference (engine/model.py:303-305,315,318-320).
-// Products are accumulated with fused multiply-adds in float32, k ascending,
-// one output element per accumulator: no reduced-precision matrix mode, no split
-// over k, and the value of an output element does not depend on M, on the tile
-// it falls in or on which other rows share the launch.
+// Products are accumulated with fused multiply-adds in float32, k ascending, in
+// blocks of 512 of k whose sums are then added up in order (with rows of 30,000
+// terms one running sum loses a digit more than the block sums do): no
+// reduced-precision matrix mode, no split over k across threads, and the value
+// of an output element does not depend on M, on the tile it falls in or on which
+// other rows share the launch.
 #include "common.h"
 #include "api.h"
 
 #define GP_BM 64
 #define GP_BN 64
 #define GP_BK 16
+#define GP_BLOCK_TILES 32  // k tiles whose sum is formed before it joins the total: 512 of k
 
 template <typename TA, typename TC>
 __global__ __launch_bounds__(256) void gemm_plain_kernel(TC* __restrict__ C, int64_t ldc,
@@ -26,12 +29,13 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(TC* __restrict__ C, int
   const int m0 = blockIdx.y * GP_BM, n0 = blockIdx.x * GP_BN;
   const int lr = tid / 4;        // tile row this thread loads
   const int lk = (tid % 4) * 4;  // first of its four k
-  float acc[4][4];
+  float acc[4][4], total[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = total[i][j] = 0.f;
 
+  int tiles_in_block = 0;
   for (int k0 = 0; k0 < K; k0 += GP_BK) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -54,6 +58,16 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(TC* __restrict__ C, int
         for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
     }
     __syncthreads();
+    if (++tiles_in_block == GP_BLOCK_TILES) {
+      tiles_in_block = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          total[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -63,7 +77,7 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(TC* __restrict__ C, int
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
       if (n >= N) continue;
-      float v = acc[i][j];
+      float v = total[i][j] + acc[i][j];
       if (bias) v += load_param(bias, b_is_f32, n);
       C[(int64_t)m * ldc + n] = from_f32<TC>(v);
     }

@@ -16,18 +16,21 @@ from typing import Dict, IO
 import numpy as np
 
 from ..config.engine_config import BLOCK_SIZE
-from .model import load_model
+from .model import TORCH_DTYPE, load_model
 from .step import StepEntry, StepRunner
 
 ROUND_TO = 64  # a request's token count is rounded up to this when the pool is sized
 
 
 class TraceReplayer:
-    def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = BLOCK_SIZE,
+    def __init__(self, model, dtype: str, max_tokens: int, block_size: int = BLOCK_SIZE,
                  max_live: int = 4, device: str = "cuda:0") -> None:
+        """`model`: a model folder, or a `Model` that is already built (then `dtype` must be its own)."""
         if ROUND_TO % block_size:
             raise ValueError(f"block_size {block_size} must divide {ROUND_TO}")
-        self.model = load_model(model_dir, dtype, device)
+        self.model = load_model(model, dtype, device) if isinstance(model, str) else model
+        if self.model.dtype != TORCH_DTYPE[dtype]:
+            raise ValueError(f"replay in {dtype} asked of a model that computes in {self.model.dtype}")
         num_blocks = max(1, -(-max_tokens // ROUND_TO) * (ROUND_TO // block_size))
         self.cache = self.model.new_cache(block_size, num_blocks, max_live)
         self.runner = StepRunner(self.model, self.cache)

@@ -35,10 +35,23 @@ def is_norm_weight(name: str) -> bool:
     return name.endswith("norm.weight") or name.endswith("layernorm.weight")
 
 
-def random_tensor(name: str, shape: Tuple[int, ...], seed: int, std: float = 0.02,
+def std_of(name: str, std) -> float:
+    """`std` is one number for every tensor, or a mapping from name endings to numbers with the
+    fallback under "" (so that, say, query and key projections can be drawn wider than the rest
+    and attention is peaked instead of flat)."""
+    if not isinstance(std, Mapping):
+        return float(std)
+    for ending, value in std.items():
+        if ending and name.endswith(ending):
+            return float(value)
+    return float(std.get("", 0.02))
+
+
+def random_tensor(name: str, shape: Tuple[int, ...], seed: int, std=0.02,
                   norm_std: float = 0.0, device: str = "cpu",
                   dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     gen = torch.Generator(device=device).manual_seed(_tensor_seed(seed, name))
+    std = std_of(name, std)
     if is_norm_weight(name):
         t = torch.ones(shape, device=device)
         if norm_std:
@@ -49,7 +62,7 @@ def random_tensor(name: str, shape: Tuple[int, ...], seed: int, std: float = 0.0
     return t.to(dtype)
 
 
-def random_weights(expected: Mapping[str, Tuple[int, ...]], seed: int, std: float = 0.02,
+def random_weights(expected: Mapping[str, Tuple[int, ...]], seed: int, std=0.02,
                    norm_std: float = 0.0, device: str = "cpu",
                    dtype: torch.dtype = torch.bfloat16) -> Dict[str, torch.Tensor]:
     return {name: random_tensor(name, tuple(shape), seed, std, norm_std, device, dtype)
@@ -61,7 +74,7 @@ class RandomWeights(Mapping):
     Two lookups of one name give equal tensors, so the same mapping can feed a model and, in a
     test, the plain implementation it is compared with."""
 
-    def __init__(self, expected: Mapping[str, Tuple[int, ...]], seed: int, std: float = 0.02,
+    def __init__(self, expected: Mapping[str, Tuple[int, ...]], seed: int, std=0.02,
                  norm_std: float = 0.0, device: str = "cuda:0", dtype: torch.dtype = torch.bfloat16) -> None:
         self.shapes = {name: tuple(shape) for name, shape in expected.items()}
         self.seed, self.std, self.norm_std, self.device, self.dtype = seed, std, norm_std, device, dtype
@@ -78,7 +91,7 @@ class RandomWeights(Mapping):
         return len(self.shapes)
 
 
-def write_model_folder(config, seed: int, out_dir: str, std: float = 0.02, norm_std: float = 0.0,
+def write_model_folder(config, seed: int, out_dir: str, std=0.02, norm_std: float = 0.0,
                        dtype: torch.dtype = torch.bfloat16) -> str:
     """Write `config.json` and `model.safetensors` for the typed `config` (any
     registered architecture's config object) with random weights."""

@@ -7,7 +7,9 @@ product package: it does not import it, uses no paging, no batching and no
 kernels, and recomputes the whole sequence for every query.
 
 Everything takes a dict of tensors keyed by checkpoint name and a plain dict of
-the config.json keys, so the same functions serve any size.
+the config.json keys, so the same functions serve any size; index tensors are made
+on the device the weights live on, so the same functions run on the CPU or, for the
+large shapes, on a GPU in float64.
 
 `dtype` is the storage dtype of activations (float64, float32 or bfloat16).
 With bfloat16 the cast points follow the reference's text: the norm's variance
@@ -68,9 +70,9 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return weight.to(in_dtype) * xw.to(in_dtype)
 
 
-def rope_inv_freq(head_dim: int, theta: float, work: torch.dtype = torch.float32) -> torch.Tensor:
+def rope_inv_freq(head_dim: int, theta: float, work: torch.dtype = torch.float32, device=None) -> torch.Tensor:
     """engine/model.py:132-135 -- 1 / theta ** (arange(0, hd, 2) / hd)."""
-    exponent = torch.arange(0, head_dim, 2, dtype=torch.int64).to(work)
+    exponent = torch.arange(0, head_dim, 2, dtype=torch.int64, device=device).to(work)
     return 1.0 / (theta ** (exponent / head_dim))
 
 
@@ -110,14 +112,14 @@ def split_heads(x: torch.Tensor, num_heads: int, head_dim: int) -> torch.Tensor:
     return x.view(n, num_heads, head_dim).transpose(0, 1)
 
 
-def allowed_keys(num_tokens: int, window: int | None) -> torch.Tensor:
+def allowed_keys(num_tokens: int, window: int | None, device=None) -> torch.Tensor:
     """Boolean (n, n): may query i see key j.
 
     engine/attention.py:474-487: key j is visible to the query at position p iff
     j <= p (and j < kv_len, which holds for a whole sequence).  With a window w
     (not in the reference) additionally p - j < w."""
-    i = torch.arange(num_tokens)[:, None]
-    j = torch.arange(num_tokens)[None, :]
+    i = torch.arange(num_tokens, device=device)[:, None]
+    j = torch.arange(num_tokens, device=device)[None, :]
     ok = j <= i
     if window is not None:
         ok = ok & ((i - j) < window)
@@ -137,8 +139,8 @@ def attention(
     nkv = k.shape[0]
     g = nh // nkv
     work = torch.float64 if q.dtype == torch.float64 else torch.float32
-    ok = allowed_keys(n, window)
-    out = torch.empty(nh, n, v.shape[-1], dtype=work)
+    ok = allowed_keys(n, window, q.device)
+    out = torch.empty(nh, n, v.shape[-1], dtype=work, device=q.device)
     for h in range(nh):
         kh = k[h // g].to(work)
         vh = v[h // g].to(work)
@@ -165,7 +167,7 @@ def self_attention(w: dict, prefix: str, cfg: dict, x: torch.Tensor, positions: 
     k = split_heads(linear(x, w[p + "k_proj.weight"], w[p + "k_proj.bias"]), nkv, hd)
     v = split_heads(linear(x, w[p + "v_proj.weight"], w[p + "v_proj.bias"]), nkv, hd)
     work = torch.float64 if x.dtype == torch.float64 else torch.float32
-    cos, sin = rope_cos_sin(rope_inv_freq(hd, rope_theta_of(cfg), work), positions, x.dtype)
+    cos, sin = rope_cos_sin(rope_inv_freq(hd, rope_theta_of(cfg), work, x.device), positions, x.dtype)
     q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
     out = attention(q, k, v, hd ** -0.5, window)
     return linear(merge_heads(out), w[p + "o_proj.weight"])
@@ -205,8 +207,9 @@ def lm_head_weight(w: dict, cfg: dict) -> torch.Tensor:
 def hidden_states(w: dict, cfg: dict, token_ids, dtype: torch.dtype = torch.float32,
                   positions=None) -> torch.Tensor:
     """Embedding gather (engine/model.py:401), every layer, final norm (:351)."""
-    ids = torch.as_tensor(token_ids, dtype=torch.long)
-    pos = torch.arange(len(ids)) if positions is None else torch.as_tensor(positions)
+    device = w["model.embed_tokens.weight"].device
+    ids = torch.as_tensor(token_ids, dtype=torch.long, device=device)
+    pos = torch.arange(len(ids), device=device) if positions is None else torch.as_tensor(positions, device=device)
     x = w["model.embed_tokens.weight"][ids].to(dtype)
     for i in range(cfg["num_hidden_layers"]):
         x = decoder_layer(w, cfg, i, x, pos)

@@ -21,7 +21,7 @@ def test_whole_prompt_and_decode(tmp_path, name, dtype):
     gen = torch.Generator().manual_seed(5)
     tokens = torch.randint(0, cfg["vocab_size"], (70,), generator=gen).tolist()
     want = plain.logits({k: v.double() for k, v in weights.items()}, cfg, tokens, torch.float64).float()
-    atol = helpers.fp32_atol(want) if dtype == "float32" else helpers.bf16_atol(want)
+    atol = helpers.bounds(dtype, want)[0]
 
     rep = TraceReplayer(folder, dtype, max_tokens=128, block_size=block)
     got = rep.step({"step": 0, "entries": [{"id": "a", "tokens": tokens, "want": list(range(70))}], "end": ["a"]})

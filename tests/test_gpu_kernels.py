@@ -274,6 +274,8 @@ def fill_pools(keys, values, tables, bs, num_blocks, dtype):
     for s, (k, v) in enumerate(zip(keys, values)):
         for p in range(k.shape[0]):
             blk = int(tables[s, p // bs])
+            if blk < 0:
+                continue  # a page the window has passed: given back, nothing of it is in the pool
             kp[blk, :, p % bs, :] = k[p].to(dtype)
             vp[blk, :, :, p % bs] = v[p].to(dtype)
     return kp, vp
@@ -407,11 +409,24 @@ def test_gemm_skinny_rope(M, nh, nkv, hd, rot, bs, Kdim, bias, k_ranges):
 
 
 # ------------------------------------------------------------------ attention
-def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=None, seed=0, ramp=None):
-    """Queries are the last q_lens[s] positions of each sequence.  Returns (got, want)."""
+def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=None, seed=0, ramp=None,
+                  holes=False):
+    """Queries are the last q_lens[s] positions of each sequence.  Returns (got, want).
+
+    `sharp`: a key position of sequence 0 that dominates the scores of its last query, or
+    (key position, index of the query within sequence 0's run).  `holes`: the pages of sequence 0
+    that lie wholly before its first query's window are given back (their table entries are -1),
+    and page 0 of the pool, which a kernel that follows a hole would land on, holds large values."""
     torch.manual_seed(seed)
     num_blocks = sum(-(-n // bs) for n in seq_lens) + 5
     tables = scattered_tables(seq_lens, bs, num_blocks, seed=seed + 1)
+    if holes:
+        assert window
+        used = set(tables.flatten().tolist()) - {-1}
+        if 0 in used:  # keep page 0 for the poison
+            tables[tables == 0] = next(b for b in range(num_blocks) if b not in used)
+        passed = max(0, seq_lens[0] - q_lens[0] - window + 1) // bs
+        tables[0, :passed] = -1
     keys = [torch.randn(n, nkv, hd) for n in seq_lens]
     values = [torch.randn(n, nkv, hd) for n in seq_lens]
     positions, tok_seq = [], []
@@ -420,12 +435,12 @@ def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=
         tok_seq += [s] * ql
     T = len(positions)
     q = torch.randn(T, nh, hd)
-    if sharp is not None:  # make one key of sequence 0 dominate its last query's scores
-        key_pos = sharp
+    if sharp is not None:  # make one key of sequence 0 dominate the scores of one of its queries
+        key_pos, q_index = sharp if isinstance(sharp, tuple) else (sharp, q_lens[0] - 1)
         direction = torch.randn(hd)
         direction /= direction.norm()
         keys[0][key_pos] = 6.0 * direction * math.sqrt(hd) ** 0.5
-        q[q_lens[0] - 1] = 6.0 * direction * math.sqrt(hd) ** 0.5
+        q[q_index] = 6.0 * direction * math.sqrt(hd) ** 0.5
     if ramp is not None:  # scores of sequence 0 climb by `ramp` (natural-log units) per key, up or down
         direction = torch.randn(hd)
         direction /= direction.norm()
@@ -436,6 +451,8 @@ def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=
     want = torch.stack([reference_attention(q[t].float(), keys[s].float(), values[s].float(), p, scale, window)
                         for t, (p, s) in enumerate(zip(positions, tok_seq))]).view(T, nh * hd)
     kp, vp = fill_pools(keys, values, tables, bs, num_blocks, DT[dtype])
+    if holes:
+        kp[0], vp[0] = 3.0e4, -3.0e4
     d = lambda x, dt=None: (x if dt is None else torch.tensor(x, dtype=dt)).to(DEV)
     out = torch.zeros(T, nh * hd, dtype=DT[dtype], device=DEV)
     qd = d(q.view(T, nh * hd).contiguous())
@@ -493,6 +510,30 @@ def test_one_far_key_stands_out(kind, key_pos, window, seen):
     # the construction works: the visible key really dominates (else the check above says little)
     if seen:
         assert want[0].abs().max() > 0.5
+
+
+@pytest.mark.parametrize("kind", ["generic", "mfma"])
+@pytest.mark.parametrize("q_len", [1, 2, 33, 64, 65])
+@pytest.mark.parametrize("which", ["first", "last"])
+@pytest.mark.parametrize("edge", ["before", "at", "unit"])
+def test_window_edges_and_given_back_pages_in_runs(kind, q_len, which, edge):
+    """A run of tokens over a window of 64 keys whose earlier pages have been given back (table
+    entries of -1; page 0 of the pool holds large numbers).  One key dominates the scores of the
+    run's first or last query: the key just before that query's window (which it must not see), the
+    first key inside it, or a key on an edge of the 32-key units the matrix-core kernel walks.  The
+    output is the plain one either way; one key too many or too few, or a read through a hole,
+    gives something far from it."""
+    nh, nkv, hd, bs, window, n = 12, 2, 128, 16, 64, 1300
+    q_index = 0 if which == "first" else q_len - 1
+    pos = n - q_len + q_index
+    start = pos - window + 1
+    key_pos = {"before": start - 1, "at": start, "unit": max(start, pos // 32 * 32)}[edge]
+    got, want = run_attention(kind, "bfloat16", nh, nkv, hd, bs, window, [n, 90], [q_len, 1],
+                              sharp=(key_pos, q_index), holes=True)
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max() <= 3e-2
+    if edge != "before":  # the construction works: the output is nearly that key's value
+        assert want[q_index].abs().max() > 0.5
 
 
 @pytest.mark.parametrize("q_len", [2, 31, 32, 33, 64, 65, 100, 128, 129, 300])

@@ -361,7 +361,8 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
 def helpers_tol(dtype, top):
     from tests import helpers
     ref = torch.tensor(top)
-    return helpers.fp32_atol(ref) * 4 if dtype == "float32" else helpers.bf16_atol(ref)
+    # the toy architecture is drawn four times wider than the tiny models: the reference's 4 ulp
+    return helpers.fp32_atol(ref) * 4 if dtype == "float32" else 4 * helpers.bf16_ulp(ref)
 
 
 # ------------------------------------------------------------------ a mixer with a cached tensor of its own

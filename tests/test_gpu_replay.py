@@ -127,7 +127,7 @@ def run_trace(folder, dtype, out_dir, max_tokens, block_size, records):
     assert proc.wait(timeout=60) == 0
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_replay_schedules_agree_with_the_plain_implementation(tmp_path, name, dtype):
     folder = helpers.make_model_folder(tmp_path, name)
@@ -138,7 +138,7 @@ def test_replay_schedules_agree_with_the_plain_implementation(tmp_path, name, dt
               for i, n in enumerate(LENGTHS)}
     want = {n: plain.logits(weights64, cfg, ids, torch.float64).float().numpy() for n, ids in tokens.items()}
     top = max(float(np.abs(w).max()) for w in want.values())
-    atol = helpers.fp32_atol(torch.tensor(top)) if dtype == "float32" else helpers.bf16_atol(torch.tensor(top))
+    atol, rms_bound = helpers.bounds(dtype, torch.tensor(top), name)
 
     trace = build_trace(tokens)
     max_tokens = peak_live_tokens(trace)
@@ -147,7 +147,7 @@ def test_replay_schedules_agree_with_the_plain_implementation(tmp_path, name, dt
     run_trace(folder, dtype, out_dir, max_tokens, helpers.TINY[name][1]["block_size"], trace.records)
 
     seen = {}  # (name, position) -> first logits seen, to compare schedules with each other
-    worst, checked = 0.0, 0
+    worst, checked, squares = 0.0, 0, 0.0
     for rec in trace.records:
         path = os.path.join(out_dir, f"{rec['step']}.f32")
         rows = trace.wanted.get(rec["step"])
@@ -158,11 +158,13 @@ def test_replay_schedules_agree_with_the_plain_implementation(tmp_path, name, dt
         for row, (req, pos) in zip(got, rows):
             err = float(np.abs(row - want[req][pos]).max())
             worst = max(worst, err)
+            squares += float(np.square(row - want[req][pos]).mean())
             assert err <= atol, f"step {rec['step']} ({req}, position {pos}): error {err:.3e} > {atol:.3e}"
             if dtype == "float32":
                 first = seen.setdefault((req, pos), row)
                 assert np.array_equal(first, row), f"step {rec['step']} ({req}, {pos}) differs between schedules"
             checked += 1
     print(f"{name} {dtype}: {len(trace.records)} steps, {checked} rows, pool for {max_tokens} tokens, "
-          f"worst error {worst:.3e} (bound {atol:.3e})")
+          f"worst error {worst:.3e} (bound {atol:.3e}), rms error {(squares / checked) ** 0.5:.3e}")
+    assert (squares / checked) ** 0.5 <= rms_bound
     assert checked > 4 * sum(LENGTHS) // 2

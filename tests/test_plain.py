@@ -254,3 +254,142 @@ def test_sampling_rules():
     assert plain.sample_from_logits(pair, 1.0, 0.49) == 0 and plain.sample_from_logits(pair, 1.0, 0.51) == 1
     # a low temperature concentrates on the maximum
     assert plain.sample_from_logits(torch.tensor([0.0, 1.0, 0.5]), 1e-3, 0.7) == 1
+
+
+# ------------------------------------------------------------------ pins that a plausible mistake fails
+def _mutated(attribute, replacement):
+    """Context manager: the plain module with one of its functions swapped for a mistaken one."""
+    import contextlib
+
+    @contextlib.contextmanager
+    def swap():
+        keep = getattr(plain, attribute)
+        setattr(plain, attribute, replacement)
+        try:
+            yield
+        finally:
+            setattr(plain, attribute, keep)
+    return swap()
+
+
+def _bias_after_rotation(w, prefix, cfg, x, positions, window):
+    """self_attention with the mistake of adding q/k bias after the rotation."""
+    nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], plain.head_dim_of(cfg)
+    p = prefix + "self_attn."
+    q = plain.split_heads(plain.linear(x, w[p + "q_proj.weight"]), nh, hd)
+    k = plain.split_heads(plain.linear(x, w[p + "k_proj.weight"]), nkv, hd)
+    v = plain.split_heads(plain.linear(x, w[p + "v_proj.weight"], w[p + "v_proj.bias"]), nkv, hd)
+    cos, sin = plain.rope_cos_sin(plain.rope_inv_freq(hd, plain.rope_theta_of(cfg), torch.float64), positions, x.dtype)
+    q = plain.apply_rope(q, cos, sin) + plain.split_heads(w[p + "q_proj.bias"][None].to(x.dtype), nh, hd)
+    k = plain.apply_rope(k, cos, sin) + plain.split_heads(w[p + "k_proj.bias"][None].to(x.dtype), nkv, hd)
+    return plain.linear(plain.merge_heads(plain.attention(q, k, v, hd ** -0.5, window)), w[p + "o_proj.weight"])
+
+
+def test_the_bias_is_added_before_the_rotation():
+    """engine/model.py:303-311: q and k get their bias, then the rotation.  Then scores depend on
+    distances only and a shift of all positions changes nothing; with the bias added after the
+    rotation the terms <R_m q, b_k> depend on the absolute position m, and the shift shows."""
+    cfg = dict(helpers.TINY_B)
+    w = {k: v.double() for k, v in plain.random_weights(cfg, 1, std=0.3, norm_std=0.1).items()}
+    ids = [5, 900, 33, 7, 512, 64, 1, 77, 3]
+    shifted = [p + 211 for p in range(len(ids))]
+    assert torch.allclose(plain.logits(w, cfg, ids, torch.float64),
+                          plain.logits(w, cfg, ids, torch.float64, positions=shifted), atol=1e-9)
+    with _mutated("self_attention", _bias_after_rotation):
+        wrong = plain.logits(w, cfg, ids, torch.float64)
+        wrong_shifted = plain.logits(w, cfg, ids, torch.float64, positions=shifted)
+    assert float((wrong - wrong_shifted).abs().max()) > 1e-3  # the mistake breaks the invariance
+
+
+def test_the_gate_goes_through_silu_and_up_does_not():
+    """engine/model.py:317-320: down(silu(gate) * up).  A strongly negative gate closes the unit
+    whatever `up` holds; had SiLU been put on `up`, the same numbers would give about -57."""
+    w = {"mlp.gate_proj.weight": torch.tensor([[-20.0]], dtype=torch.float64),
+         "mlp.up_proj.weight": torch.tensor([[3.0]], dtype=torch.float64),
+         "mlp.down_proj.weight": torch.tensor([[1.0]], dtype=torch.float64)}
+    y = plain.swiglu_mlp(w, "", torch.ones(1, 1, dtype=torch.float64))
+    assert abs(float(y)) < 1e-6
+    assert abs(float(plain.silu(torch.tensor(3.0, dtype=torch.float64)) * -20.0)) > 50  # what the swap would give
+    # and an open gate of 1.0 scales `up` by silu(1) = 1 / (1 + e^-1)
+    w["mlp.gate_proj.weight"] = torch.tensor([[1.0]], dtype=torch.float64)
+    assert abs(float(plain.swiglu_mlp(w, "", torch.ones(1, 1, dtype=torch.float64))) - 3.0 / (1 + math.exp(-1))) < 1e-12
+
+
+def test_one_layer_one_token_is_a_closed_chain():
+    """engine/model.py:340-351 for one token (whose attention is its own value vector, softmax of
+    one score being 1): h1 = e + Wo (Wv n1(e) + bv); h2 = h1 + MLP(n2(h1)); logits = head nf(h2).
+    Pins the arrangement: each norm feeds its branch only, the residual carries the un-normed sum,
+    the final norm comes before the head.  A post-norm block, a norm on the residual, or a
+    missing final norm all give other numbers."""
+    cfg = dict(helpers.TINY_B, num_hidden_layers=1)
+    w = {k: v.double() for k, v in plain.random_weights(cfg, 5, std=0.2, norm_std=0.2).items()}
+    p, eps, tok = "model.layers.0.", cfg["rms_norm_eps"], 321
+    e = w["model.embed_tokens.weight"][tok][None]
+    n1 = plain.rms_norm(e, w[p + "input_layernorm.weight"], eps)
+    value = n1 @ w[p + "self_attn.v_proj.weight"].t() + w[p + "self_attn.v_proj.bias"]  # [1, nkv * hd]
+    nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    per_head = value.view(nkv, hd).repeat_interleave(nh // nkv, dim=0).reshape(1, nh * hd)  # kv head j serves heads j*g..
+    h1 = e + per_head @ w[p + "self_attn.o_proj.weight"].t()
+    n2 = plain.rms_norm(h1, w[p + "post_attention_layernorm.weight"], eps)
+    gate, up = n2 @ w[p + "mlp.gate_proj.weight"].t(), n2 @ w[p + "mlp.up_proj.weight"].t()
+    h2 = h1 + (gate * torch.sigmoid(gate) * up) @ w[p + "mlp.down_proj.weight"].t()
+    want = plain.rms_norm(h2, w["model.norm.weight"], eps) @ w["lm_head.weight"].t()
+    got = plain.logits(w, cfg, [tok], torch.float64)
+    assert torch.allclose(got, want, atol=1e-10)
+    # the branches matter in this check: without them the logits are far away
+    bare = plain.rms_norm(e, w["model.norm.weight"], eps) @ w["lm_head.weight"].t()
+    assert float((bare - want).abs().max()) > 0.1
+
+
+def test_the_window_rule():
+    """Not in the reference (every layer there sees every earlier key): layers from
+    `max_window_layers` on look back `sliding_window` keys.  Parity unpinned; what is pinned is
+    that the rule does what it says: a window as long as the sequence changes nothing, the
+    layers below `max_window_layers` are not windowed, a window of one sees only the token itself."""
+    cfg = dict(helpers.TINY_C)
+    assert [plain.layer_window(cfg, i) for i in range(4)] == [None, None, 24, 24]
+    assert plain.layer_window(dict(cfg, use_sliding_window=False), 3) is None
+    w = {k: v.double() for k, v in plain.random_weights(cfg, 2, std=0.2).items()}
+    ids = list(range(3, 33))
+    full = plain.logits(w, dict(cfg, use_sliding_window=False), ids, torch.float64)
+    assert torch.allclose(plain.logits(w, dict(cfg, sliding_window=len(ids)), ids, torch.float64), full, atol=1e-12)
+    assert not torch.allclose(plain.logits(w, cfg, ids, torch.float64), full, atol=1e-6)
+    assert torch.allclose(plain.logits(w, cfg, ids, torch.float64)[:24], full[:24], atol=1e-12)  # the first 24 see all
+    q = torch.randn(2, 5, 8, dtype=torch.float64)
+    v = torch.randn(1, 5, 8, dtype=torch.float64)
+    out = plain.attention(q, torch.randn(1, 5, 8, dtype=torch.float64), v, 0.3, window=1)
+    assert torch.allclose(out[0], v[0]) and torch.allclose(out[1], v[0])
+
+
+def test_the_peaked_model_shows_mistakes_far_beyond_the_bfloat16_bound(tmp_path):
+    """The bfloat16 tests can fail: on model E (tests/helpers.py) the logits move by more than ten
+    times the bound they are held to when the rotation is dropped, when attention is flattened,
+    when the window is off by one, when the bias comes after the rotation, and when query heads
+    are paired with the wrong key/value head.  (With weights N(0, 0.02) everywhere, as in models
+    A to D, the same mistakes move the logits by less than the bound.)"""
+    folder = helpers.make_model_folder(tmp_path, "E")
+    cfg, w = helpers.read_folder_plain(folder)
+    w = {k: v.double() for k, v in w.items()}
+    ids = torch.randint(0, cfg["vocab_size"], (130,), generator=torch.Generator().manual_seed(11)).tolist()
+    base = plain.logits(w, cfg, ids, torch.float64)
+    bound = helpers.bf16_atol(base, "E")
+
+    def moved(logits):
+        return float((logits - base).abs().max()) / bound
+
+    with _mutated("apply_rope", lambda x, cos, sin: x):
+        assert moved(plain.logits(w, cfg, ids, torch.float64)) > 10
+    real_attention = plain.attention
+    with _mutated("attention", lambda q, k, v, scale, window=None: real_attention(torch.zeros_like(q), k, v, scale, window)):
+        assert moved(plain.logits(w, cfg, ids, torch.float64)) > 10
+    for off in (-1, 1):
+        assert moved(plain.logits(w, dict(cfg, sliding_window=cfg["sliding_window"] + off), ids, torch.float64)) > 10
+    with _mutated("self_attention", _bias_after_rotation):
+        assert moved(plain.logits(w, cfg, ids, torch.float64)) > 10
+    # heads paired the other way round: query head h reads key/value head h % nkv instead of h // g
+    def interleaved(q, k, v, scale, window=None):
+        nh, nkv = q.shape[0], k.shape[0]
+        order = [(h % nkv) * (nh // nkv) + h // nkv for h in range(nh)]
+        return real_attention(q[order], k, v, scale, window)[[order.index(h) for h in range(nh)]]
+    with _mutated("attention", interleaved):
+        assert moved(plain.logits(w, cfg, ids, torch.float64)) > 10
