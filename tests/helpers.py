@@ -100,14 +100,17 @@ def bf16_ulp(reference_logits: torch.Tensor) -> float:
 # The reference states its reduced-precision parity as 4 ulp of the logits' binade
 # (tests/test_parity_fp16.py:161-163).  With flat attention (weights N(0, 0.02): scores a few
 # hundredths wide) this engine stays within 1 ulp, so those models are held to 2 ulp at the worst
-# logit and a quarter of an ulp in the root mean square.  Model E's scores are some ten units wide:
+# logit.  Model E's scores are some ten units wide:
 # rounding q and k to bfloat16 alone moves a score by several hundredths and a softmax weight by
-# several per cent, whatever the kernel, so E keeps the reference's 4 ulp (and three quarters in the
-# root mean square); its job is the other direction: a wrong kernel moves its logits by 45 times that.
+# several per cent, whatever the kernel, so E keeps the reference's 4 ulp; its job is the other direction: a wrong kernel moves its logits by 45 times that.
 # The same holds at the real layer sizes ("wide"): with hidden widths of 1,536 to 8,192 the scores of
 # N(0, 0.02) weights are one to three units wide by themselves.
 BF16_MAX_ULPS = {"E": 4.0, "wide": 4.0}
-BF16_RMS_ULPS = {"E": 0.75, "wide": 0.75}
+# The root mean square over all logits is held to a share of the largest logit instead of its
+# binade (a bound that halves when the largest logit drops from 1.01 to 0.99 says little about an
+# average): 2**-9 of it, half a unit in the last place of a bfloat16 number of that size, for the
+# flat models (observed: at most 0.55 of that), and 2.5 times as much where attention is peaked.
+BF16_RMS_SHARE = {"E": 2.5, "wide": 2.5}
 
 
 def bf16_atol(reference_logits: torch.Tensor, name: str = "") -> float:
@@ -115,7 +118,8 @@ def bf16_atol(reference_logits: torch.Tensor, name: str = "") -> float:
 
 
 def bf16_rms_bound(reference_logits: torch.Tensor, name: str = "") -> float:
-    return BF16_RMS_ULPS.get(name, 0.25) * bf16_ulp(reference_logits)
+    top = max(float(torch.as_tensor(reference_logits).abs().max()), 1e-6)
+    return BF16_RMS_SHARE.get(name, 1.0) * 2.0 ** -9 * top
 
 
 def bounds(dtype: str, reference_logits: torch.Tensor, name: str = ""):

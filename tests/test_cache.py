@@ -24,6 +24,7 @@ def check_allocator(alloc: BlockAllocator):
     assert not set(free) & set(held)
     assert sorted(free + held) == list(range(alloc.num_blocks))
     assert alloc.num_free + alloc.num_allocated == alloc.num_blocks
+    alloc.audit()  # the allocator's own check of the same, page by page
 
 
 def test_allocator_invariants_under_random_operations():
@@ -199,3 +200,49 @@ def test_manager_under_random_requests():
     for seq in live:
         cache.free_sequence(seq)
     assert cache.free_blocks() == (12, 7)
+
+
+def test_a_page_cannot_come_back_twice_or_from_a_stranger():
+    alloc = BlockAllocator(4, 4)
+    alloc.create_sequence(0)
+    alloc.create_sequence(1)
+    alloc.append_tokens(0, 8)
+    alloc.append_tokens(1, 4)
+    page = alloc.block_table(1)[0]
+    with pytest.raises(AssertionError):
+        alloc._give_back(0, page)  # sequence 0 does not hold it
+    alloc.free_sequence(1)
+    with pytest.raises(AssertionError):
+        alloc._give_back(1, page)  # it is free already
+    alloc.audit()
+    assert alloc.num_free == 2 and alloc.free_block_ids() == (3, page)
+
+
+def test_the_table_array_is_the_table():
+    alloc = BlockAllocator(6, 2)
+    alloc.create_sequence(3)
+    alloc.append_tokens(3, 5)
+    view = alloc.table_array(3)
+    assert list(view) == list(alloc.block_table(3)) == [0, 1, 2]
+    alloc.release_before(3, 2)
+    assert list(view) == [HOLE, 1, 2]  # not a copy: the step's staging buffer reads the live table
+
+
+def test_pages_hold_what_the_mixer_declares():
+    from paged_attention_engine_amd.cache import PAGE, PagedTensor, bytes_of_one_page_everywhere
+    import torch
+
+    latent = PagedSpec((PagedTensor("latent", (PAGE, 24)),))
+    kv = attention_pages(2, 16, window=6)
+    assert kv.elements_per_token() == 2 * 2 * 16 and latent.elements_per_token() == 24
+    assert [t.shape(4) for t in kv.tensors] == [(2, 4, 16), (2, 16, 4)]
+    # stops 0 and 1 share a group (same spec), stop 2 has its own; the byte arithmetic counts every stop
+    assert bytes_of_one_page_everywhere([kv, kv, latent, None], 4, torch.bfloat16) == (2 * 64 + 24) * 4 * 2
+    cache = CacheManager([kv, kv, latent, None], [None] * 4, block_size=4, num_blocks=5, num_slots=2, device=None)
+    assert [g.entries for g in cache.groups] == [[0, 1], [2]]
+    assert cache.storage_bytes() == 5 * (2 * 64 + 24) * 4 * 4  # float32 by default
+    assert cache.padding_page(0) == 5 and cache.padding_slot == 2
+    with pytest.raises(ValueError):
+        PagedTensor("x", (3, 4))           # no PAGE axis
+    with pytest.raises(ValueError):
+        PagedSpec((PagedTensor("a", (PAGE,)), PagedTensor("a", (PAGE, 2))))  # one name twice

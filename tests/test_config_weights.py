@@ -181,3 +181,70 @@ def test_sharded_folder(tmp_path):
         json.dump({"weight_map": {"a": "model-00001-of-00002.safetensors", "b": "model-00002-of-00002.safetensors"}}, handle)
     out = pae.load_weights(folder, {"a": (2,), "b": (3,)})
     assert torch.equal(out["a"], torch.ones(2)) and torch.equal(out["b"], torch.zeros(3))
+
+
+# ------------------------------------------------------------------ pool sizing, random weights, shards
+def test_the_pool_is_sized_once_in_pages_or_bytes_or_a_share_of_free_memory():
+    from paged_attention_engine_amd.config.engine_config import NUM_GPU_BLOCKS, EngineConfig
+
+    asked = []
+
+    def free():
+        asked.append(1)
+        return 1000
+
+    assert EngineConfig().pages(100, free) == NUM_GPU_BLOCKS
+    assert EngineConfig(num_blocks=7).pages(100, free) == 7
+    assert EngineConfig(kv_bytes=1050).pages(100, free) == 10 and not asked
+    assert EngineConfig(fill_hbm=0.55).pages(100, free) == 5 and asked
+    with pytest.raises(ValueError, match="once"):
+        EngineConfig(num_blocks=4, kv_bytes=100)
+    with pytest.raises(ValueError):
+        EngineConfig(fill_hbm=1.5)
+    with pytest.raises(ValueError, match="one page"):
+        EngineConfig(kv_bytes=99).pages(100, free)
+
+
+def test_random_weights_are_drawn_at_the_lookup_and_repeat():
+    from paged_attention_engine_amd.weights import RandomWeights
+
+    shapes = {"a.q_proj.weight": (6, 4), "a.input_layernorm.weight": (4,), "b.weight": (3, 3)}
+    drawn = RandomWeights(shapes, seed=5, std={"": 0.02, "q_proj.weight": 0.5}, norm_std=0.1, device="cpu")
+    assert sorted(drawn) == sorted(shapes) and len(drawn) == 3
+    first, again = drawn["a.q_proj.weight"], drawn["a.q_proj.weight"]
+    assert first is not again and torch.equal(first, again) and first.dtype == torch.bfloat16
+    assert float(first.float().std()) > 0.2 > float(drawn["b.weight"].float().std())  # the wider ending applies
+    assert float((drawn["a.input_layernorm.weight"].float() - 1).abs().max()) < 0.5
+    assert not torch.equal(first, RandomWeights(shapes, seed=6, device="cpu")["a.q_proj.weight"])
+    with pytest.raises(KeyError):
+        drawn["c"]
+    assert drawn.get("c") is None
+
+
+def test_an_index_that_names_what_a_shard_lacks_is_a_weights_error(tmp_path):
+    import json
+
+    from paged_attention_engine_amd.weights import load_weights, save_file
+
+    save_file({"a": torch.zeros(2, 2)}, str(tmp_path / "part1.safetensors"))
+    index = {"weight_map": {"a": "part1.safetensors", "b": "part1.safetensors"}}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    with pytest.raises(pae.WeightsError, match="b \\(not in part1.safetensors\\)") as err:
+        load_weights(str(tmp_path), {"a": (2, 2), "b": (2, 2)})
+    assert err.value.missing == ("b",)
+    index["weight_map"]["b"] = "part2.safetensors"
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    with pytest.raises(pae.WeightsError, match="part2.safetensors"):
+        load_weights(str(tmp_path), {"a": (2, 2), "b": (2, 2)})
+
+
+def test_loaded_weights_are_views_of_the_file(tmp_path):
+    from paged_attention_engine_amd.weights import load_weights, save_file
+
+    save_file({"a": torch.arange(6, dtype=torch.float32).view(2, 3), "h": torch.ones(2, dtype=torch.float16)},
+              str(tmp_path / "model.safetensors"))
+    weights = load_weights(str(tmp_path), {"a": (2, 3), "h": (2,)})
+    assert not isinstance(weights, dict) and sorted(weights) == ["a", "h"]
+    assert torch.equal(weights["a"], torch.arange(6, dtype=torch.float32).view(2, 3))
+    assert weights["h"].dtype == torch.float32  # half precision is widened, nothing else is copied
+    assert weights.get("zzz") is None

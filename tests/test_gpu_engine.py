@@ -170,11 +170,17 @@ def test_scheduler_runs_the_baseline_workloads(tmp_path, name, budget, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_preemption_with_recompute_is_transparent(tmp_path, dtype):
+@pytest.mark.parametrize("name", ["A", "D", "E"])
+def test_preemption_with_recompute_is_transparent(tmp_path, name, dtype):
     """Four requests that grow far beyond what admission charged them, in a pool that cannot
-    hold them all: some are evicted and replayed, and every token equals the run alone."""
-    folder = helpers.make_model_folder(tmp_path, "A")
-    cfg = helpers.TINY_A
+    hold them all: some are evicted and replayed, and every token equals the run alone.  Models D
+    and E take the serving kernels (matrix-core attention over pages that were given back and
+    taken again, windows with holes, the few-row products); E's attention is peaked.  In
+    bfloat16, where a replay sums in another order than the first run, a request's tokens may part
+    from the run alone only at a token where the plain logits nearly tie."""
+    folder = helpers.make_model_folder(tmp_path, name)
+    cfg, weights = helpers.read_folder_plain(folder)
+    weights64 = {k: v.double() for k, v in weights.items()}
     model = pae.load_model(folder, dtype)
     requests = [pae.Request(f"g{i}", tuple(tokens_of(cfg, 4, 50 + i)), 60) for i in range(4)]
     alone = {}
@@ -189,16 +195,25 @@ def test_preemption_with_recompute_is_transparent(tmp_path, dtype):
     assert small.events_of(pae.EventKind.PREEMPT) and small.events_of(pae.EventKind.RECOMPUTE)
     if dtype == "float32":
         assert out == alone
-    cfg2, weights = helpers.read_folder_plain(folder)
     for r in requests:  # replayed or not, every logit row is that of the plain implementation
         seq = small.finished[r.request_id]
         assert len(seq.step_logits) == 60
-        check_teacher_forced(cfg2, weights, r.prompt_token_ids, seq.generated, torch.stack(seq.step_logits), dtype, False)
-    assert small.cache.free_blocks() == (6,)
+        check_teacher_forced(cfg, weights, r.prompt_token_ids, seq.generated, torch.stack(seq.step_logits), dtype,
+                             False, name=name)
+        got, ref = out[r.request_id], alone[r.request_id]
+        if got != ref:
+            k = next(i for i in range(60) if got[i] != ref[i])
+            history = list(r.prompt_token_ids) + list(got[:k])
+            row = plain.logits(weights64, cfg, history, torch.float64)[-1]
+            top2 = row.topk(2).values
+            bound = atol_for(dtype, row, name)
+            assert float(top2[0] - top2[1]) <= 2 * bound, f"{r.request_id}: token {k} differs at a clear margin"
+            assert {got[k], ref[k]} <= set(row.topk(4).indices.tolist())
+    assert all(n == 6 for n in small.cache.free_blocks())
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,num_blocks", [("B", 60), ("B", 14), ("C", 40)])
+@pytest.mark.parametrize("name,num_blocks", [("B", 60), ("B", 14), ("C", 40), ("D", 7), ("E", 7)])
 def test_overlapped_steps_give_the_tokens_of_single_steps(tmp_path, name, num_blocks, dtype):
     """`run_to_completion` launches the next step before it has seen the current one's tokens
     (the sampled ids go from step to step on the device).  Greedy and temperature requests,
@@ -213,8 +228,8 @@ def test_overlapped_steps_give_the_tokens_of_single_steps(tmp_path, name, num_bl
                 for i, (n, new, temp) in enumerate(shapes)]
 
     def run(overlap):
-        engine = pae.Engine(model, dtype=dtype, block_size=8, num_blocks=num_blocks, max_num_seqs=4,
-                            max_num_batched_tokens=32)
+        engine = pae.Engine(model, dtype=dtype, block_size=helpers.TINY[name][1]["block_size"] if name in "DE" else 8,
+                            num_blocks=num_blocks, max_num_seqs=4, max_num_batched_tokens=32)
         for r in requests:
             assert engine.add_request(r)
         assert engine.scheduler.can_overlap()
@@ -227,7 +242,7 @@ def test_overlapped_steps_give_the_tokens_of_single_steps(tmp_path, name, num_bl
     assert single[0] == overlapped[0] and single[1] == overlapped[1]
     assert all(len(single[0][r.request_id]) == r.max_new_tokens for r in requests)
     assert all(0 <= t < cfg["vocab_size"] for tokens in overlapped[0].values() for t in tokens)
-    if num_blocks == 14:
+    if num_blocks in (14, 7):
         assert any(kind is pae.EventKind.PREEMPT for _, kind, _, _ in single[1])
     assert overlapped[2] > 0  # decode steps were replayed graphs fed from the device
 

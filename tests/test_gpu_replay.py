@@ -127,9 +127,21 @@ def run_trace(folder, dtype, out_dir, max_tokens, block_size, records):
     assert proc.wait(timeout=60) == 0
 
 
+@pytest.mark.parametrize("name", ["D", "E"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_with_pages_of_32_tokens(tmp_path, name, dtype):
+    """The same trace with twice as many tokens to a page as the models' own tests use: the
+    matrix-core attention kernels walk pages of 32, windows pass them half as often."""
+    replay_and_compare(tmp_path, name, dtype, 32)
+
+
 @pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_replay_schedules_agree_with_the_plain_implementation(tmp_path, name, dtype):
+    replay_and_compare(tmp_path, name, dtype, helpers.TINY[name][1]["block_size"])
+
+
+def replay_and_compare(tmp_path, name, dtype, block_size):
     folder = helpers.make_model_folder(tmp_path, name)
     cfg, weights = helpers.read_folder_plain(folder)
     weights64 = {k: v.double() for k, v in weights.items()}
@@ -144,7 +156,7 @@ def test_replay_schedules_agree_with_the_plain_implementation(tmp_path, name, dt
     max_tokens = peak_live_tokens(trace)
     assert max_tokens <= 4 * 192  # four live requests at most
     out_dir = str(tmp_path / "out")
-    run_trace(folder, dtype, out_dir, max_tokens, helpers.TINY[name][1]["block_size"], trace.records)
+    run_trace(folder, dtype, out_dir, max_tokens, block_size, trace.records)
 
     seen = {}  # (name, position) -> first logits seen, to compare schedules with each other
     worst, checked, squares = 0.0, 0, 0.0
