@@ -7,14 +7,14 @@ from .config import (ConfigError, EngineConfig, known_architectures, read_config
                      register_architecture)
 from .engine.executor import ModelExecutor
 from .engine.llm import Engine, GenerationResult
-from .engine.model import Model, expected_tensors, load_model
+from .engine.model import Model, expected_tensors, load_model, random_model
 from .engine.scheduler import (Event, EventKind, Request, Scheduler, Sequence, SequenceStatus, StepResult,
                                is_admissible)
 from .engine.step import StepEntry, StepRunner
-from .weights import WeightsError, load_weights, write_model_folder
+from .weights import RandomWeights, WeightsError, load_weights, write_model_folder
 
 __all__ = ["BlockAllocator", "CacheManager", "ConfigError", "Engine", "EngineConfig", "Event", "EventKind",
            "GenerationResult", "Model", "ModelExecutor", "Request", "Scheduler", "Sequence", "SequenceStatus",
            "StepEntry", "StepResult", "StepRunner", "WeightsError", "expected_tensors", "is_admissible",
-           "known_architectures", "load_model", "load_weights", "read_config", "read_config_dict",
-           "register_architecture", "write_model_folder"]
+           "known_architectures", "load_model", "load_weights", "random_model", "read_config", "read_config_dict",
+           "register_architecture", "write_model_folder", "RandomWeights"]
