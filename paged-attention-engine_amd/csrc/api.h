@@ -11,6 +11,11 @@ int pae_device_arch(char* out, int cap);  // "gfx950" on the card the kernels ar
 
 int pae_embedding(int dtype, void* out, const void* table, const int* ids, int num_tokens, int hidden,
                   int vocab, float scale, hipStream_t stream);
+int pae_embedding_rows(int dtype, void* residual, const void* table, const int* ids, int num_tokens, int hidden,
+                       int vocab, float scale, void* next_rows, const void* next_w, int next_w_is_f32,
+                       float* next_stats, hipStream_t stream);
+int pae_scaled_rows(void* out, const void* rows, const float* row_stats, int row_stat_tiles, float eps, int num_rows,
+                    int hidden, hipStream_t stream);
 int pae_logits_finish(float* logits, int64_t n, float scale, float cap, hipStream_t stream);
 int pae_add_rmsnorm(int dtype, void* residual, const void* delta, int parts, int64_t part_stride,
                     const void* weight, int w_is_f32, float eps, const int* rows, void* out, int num_rows,
@@ -27,14 +32,16 @@ int pae_gemm_plain(int in_dtype, int out_dtype, void* C, int64_t ldc, const void
                    const void* bias, int b_is_f32, int M, int N, int K, hipStream_t stream);
 int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
                     const void* bias, int b_is_f32, int M, int N, int K, int splits, int64_t part_stride,
-                    float* ticket_parts, int* ticket_counters, hipStream_t stream);
+                    float* ticket_parts, int* ticket_counters, const float* row_stats, int row_stat_tiles,
+                    float row_eps, void* next_rows, int64_t ld_next, const void* next_w, int next_w_is_f32,
+                    float* next_stats, hipStream_t stream);
 int pae_skinny_ticket_slots(int M, int N);
 int64_t pae_skinny_ticket_floats(int M, int N, int splits);
 int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int64_t lda, const void* W, const void* bias,
                          int b_is_f32, int M, int K, int nh, int nkv, int hd, int rot, const float* cos_sin,
                          const int* positions, const int* tok_seq, const int* block_tables, int max_blocks, int bs,
                          void* k_cache, void* v_cache, int splits, float* ticket_parts, int* ticket_counters,
-                         hipStream_t stream);
+                         const float* row_stats, int row_stat_tiles, float row_eps, hipStream_t stream);
 int pae_paged_attention_generic(int dtype, void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                 const void* k_cache, const void* v_cache, const int* positions,
                                 const int* tok_seq, const int* block_tables, int max_blocks, int bs,

@@ -34,6 +34,91 @@ extern "C" int pae_embedding(int dtype, void* out, const void* table, const int*
   return pae_check_launch("embedding");
 }
 
+// The embedding for a step whose first norm is folded into the products around it (see
+// gemm_skinny.hip): beside the float32 rows, bfloat16(row * next_w) for the first product and the
+// shares of every row's sum of squares, one per 16 columns.
+template <typename T>
+__global__ void embedding_rows_kernel(float* __restrict__ out, const T* __restrict__ table, const int* __restrict__ ids,
+                                      int hidden, float scale, bf16_t* __restrict__ next_rows,
+                                      const void* __restrict__ next_w, int next_w_is_f32,
+                                      float* __restrict__ next_stats) {
+  // four lanes to a tile of 16 columns, four columns each; their squares meet through two shuffles
+  const int t = blockIdx.x, tiles = (hidden + 15) / 16;
+  const T* row = table + (int64_t)ids[t] * hidden;
+  const int quarter = threadIdx.x % 4;
+  for (int tile = threadIdx.x / 4; tile < (tiles + 63) / 64 * 64; tile += blockDim.x / 4) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = 16 * tile + 4 * quarter + j;
+      if (tile < tiles && i < hidden) {
+        const float v = scale * to_f32(row[i]);
+        out[(int64_t)t * hidden + i] = v;
+        next_rows[(int64_t)t * hidden + i] = __float2bfloat16(v * load_param(next_w, next_w_is_f32, i));
+        ss += v * v;
+      }
+    }
+    ss += __shfl_xor(ss, 1);
+    ss += __shfl_xor(ss, 2);
+    if (quarter == 0 && tile < tiles) next_stats[(int64_t)t * tiles + tile] = ss;
+  }
+}
+
+extern "C" int pae_embedding_rows(int dtype, void* residual, const void* table, const int* ids, int num_tokens,
+                                  int hidden, int vocab, float scale, void* next_rows, const void* next_w,
+                                  int next_w_is_f32, float* next_stats, hipStream_t stream) {
+  PAE_REQUIRE(num_tokens >= 0 && hidden > 0 && vocab > 0, "embedding_rows: bad sizes T=%d H=%d V=%d", num_tokens, hidden, vocab);
+  PAE_REQUIRE(next_rows && next_w && next_stats, "embedding_rows: the next product's rows, weight and sums are missing");
+  if (num_tokens == 0) return 0;
+  if (dtype == PAE_F32)
+    embedding_rows_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)residual, (const float*)table, ids, hidden, scale,
+                                                                 (bf16_t*)next_rows, next_w, next_w_is_f32, next_stats);
+  else if (dtype == PAE_BF16)
+    embedding_rows_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((float*)residual, (const bf16_t*)table, ids, hidden, scale,
+                                                                  (bf16_t*)next_rows, next_w, next_w_is_f32, next_stats);
+  else
+    return pae_fail("embedding_rows: unknown dtype code %d", dtype);
+  return pae_check_launch("embedding_rows");
+}
+
+// out[m] = bfloat16(rows[m] * rsqrt(sum(row_stats[m]) / hidden + eps)): rows whose scale is still
+// owed (see gemm_skinny.hip), paid here for a part that wants plain normalised activations.  The
+// shares are added in the order the products add them.
+__global__ void scaled_rows_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ rows,
+                                   const float* __restrict__ row_stats, int tiles, float eps, int hidden) {
+  __shared__ float s_scale;
+  const int m = blockIdx.x;
+  if (threadIdx.x < PAE_WAVE) {
+    // the order in which the products add the shares (gemm_skinny.hip, row_scale_of)
+    const int lane = threadIdx.x, g4 = lane / 16;
+    const float* shares = row_stats + (int64_t)m * tiles;
+    float sum = 0.f;
+    for (int base = 0; base < tiles; base += 128)
+      for (int u = 0; u < 8; ++u) {
+        const int t = base + 16 * u + 4 * g4;
+        float v[4];
+        for (int i = 0; i < 4; ++i) v[i] = t + i < tiles ? shares[t + i] : 0.f;
+        sum += (v[0] + v[1]) + (v[2] + v[3]);
+      }
+    sum += __shfl_xor(sum, 16);
+    sum += __shfl_xor(sum, 32);
+    if (lane == 0) s_scale = rsqrtf(sum / (float)hidden + eps);
+  }
+  __syncthreads();
+  const float scale = s_scale;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    out[(int64_t)m * hidden + i] = __float2bfloat16(__bfloat162float(rows[(int64_t)m * hidden + i]) * scale);
+}
+
+extern "C" int pae_scaled_rows(void* out, const void* rows, const float* row_stats, int row_stat_tiles, float eps,
+                               int num_rows, int hidden, hipStream_t stream) {
+  PAE_REQUIRE(num_rows >= 0 && hidden > 0 && row_stat_tiles > 0 && row_stats, "scaled_rows: bad sizes rows=%d H=%d tiles=%d",
+              num_rows, hidden, row_stat_tiles);
+  if (num_rows == 0) return 0;
+  scaled_rows_kernel<<<num_rows, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)rows, row_stats, row_stat_tiles, eps, hidden);
+  return pae_check_launch("scaled_rows");
+}
+
 // ---------------------------------------------------------------- logits: scale and soft cap
 // x = scale * x, then, with cap > 0, x = cap * tanh(x / cap).  Not part of the reference's model
 // (its logits are the head product as it is); an architecture's plan may ask for either.

@@ -29,6 +29,71 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 #define EPI_F32 1
 #define EPI_SWIGLU 2
 #define EPI_ROPE 3
+#define EPI_RESIDUAL 4
+
+// RMS normalisation folded into the products around it, so that a decode step needs no norm
+// kernel between them.  norm(x) W^T = rsqrt(mean(x^2) + eps) * ((x * w_norm) W^T): the scale is one
+// number per row and can be applied to the finished sums.
+//
+// Producer (EPI_RESIDUAL, the product that ends a residual branch): the sums of all k ranges are
+// added into the float32 residual in place; the same tile is written again as
+// bfloat16(residual * w_next), the rows the next product multiplies, and the tile's share of every
+// row's sum of squares goes to next_stats[m][16-column tile].
+// Consumer (any epilogue): `row_stats` holds those shares for the rows of A; every lane adds up
+// its row's shares in a fixed order (the same in every workgroup, so all columns of a row get the
+// same scale) and multiplies its sums by rsqrt(total / K + eps) before bias, rotation or gate.
+struct SkinnyNorm {
+  const float* row_stats;  // [M][row_stat_tiles] or null: A's rows are used as they are
+  int row_stat_tiles;
+  float eps;
+  bf16_t* next_rows;       // EPI_RESIDUAL: [M][ld_next] bfloat16(residual * next_w)
+  int64_t ld_next;
+  const void* next_w;      // [N] weight of the norm that follows
+  int next_w_is_f32;
+  float* next_stats;       // [M][(N + 15) / 16]
+};
+
+// rsqrt(mean of squares + eps) of row m of A from the shares the producer left.  The four lanes
+// that hold row m (g4 = 0..3) read the shares 16 bytes at a time, all reads of a batch of up to
+// 128 shares in flight at once (a loop that adds one share after the other waits out the memory's
+// latency once per share), add theirs in index order and then each other's: the same order in every
+// workgroup, so every column of a row is scaled by the same number.
+__device__ __forceinline__ float row_scale_of(const SkinnyNorm& norm, int m, int g4, float inv_width) {
+  const float* shares = norm.row_stats + (int64_t)m * norm.row_stat_tiles;
+  const int tiles = norm.row_stat_tiles;
+  const bool aligned = tiles % 4 == 0;  // rows of shares then start on 16-byte boundaries
+  float sum = 0.f;
+  for (int base = 0; base < tiles; base += 128) {
+    f32x4 part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int t = base + 16 * u + 4 * g4;
+      if (aligned && t + 4 <= tiles) {
+        part[u] = *reinterpret_cast<const f32x4*>(shares + t);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) part[u][i] = t + i < tiles ? shares[t + i] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) sum += (part[u][0] + part[u][1]) + (part[u][2] + part[u][3]);
+  }
+  sum += __shfl_xor(sum, 16);
+  sum += __shfl_xor(sum, 32);
+  return rsqrtf(sum * inv_width + norm.eps);
+}
+
+// The scales of this lane's rows of A (row 16 mt + lane % 16 of column tile mt), 1 without a folded
+// norm.  Asked for at the start of a kernel, so that the shares arrive while the products run.
+template <int MT>
+__device__ __forceinline__ void row_scales(float (&scale)[MT], const SkinnyNorm& norm, int M, int K) {
+  const int lane = threadIdx.x % PAE_WAVE;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + lane % 16;
+    scale[mt] = norm.row_stats ? row_scale_of(norm, m < M ? m : M - 1, lane / 16, 1.0f / (float)K) : 1.0f;
+  }
+}
 
 // What the rotating epilogue needs beside the product: the head geometry, the
 // rotation's frequencies, every row's position and sequence, and the paged cache.
@@ -71,7 +136,8 @@ template <int MT, int RT, int EPI>
 __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int tile_base, int only_mt,
                                                 void* __restrict__ out, int64_t ldc, const void* __restrict__ bias,
                                                 int b_is_f32, int M, int N, int split, int64_t part_stride,
-                                                const SkinnyRope& rope) {
+                                                const SkinnyRope& rope, const SkinnyNorm& norm,
+                                                const float (&scale)[MT]) {
   const int lane = threadIdx.x % PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
   if (EPI == EPI_ROPE) {
@@ -97,7 +163,7 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
         for (int i = 0; i < 4; ++i) {
           // the projection is rounded to bfloat16 before the rotation, as where the two are separate kernels
           const float own = __bfloat162float(__float2bfloat16(
-              acc[rt][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f)));
+              acc[rt][mt][i] * scale[mt] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f)));
           const float other = __shfl_xor(own, 32);  // in every lane
           float o = own;
           if (rotated) {
@@ -143,12 +209,44 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
         s16x4 v;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float own = acc[rt][mt][i];
-          const float up = __shfl_xor(own, 32);  // in every lane
+          const float own = acc[rt][mt][i] * scale[mt];
+          const float up = __shfl_xor(own, 32);  // in every lane (the same row of A, so the same scale)
           v[i] = to_bf16_bits(own / (1.0f + expf(-own)) * up);
         }
         if (g4 < 2 && j < N / 2)  // N counts gate and up rows
           *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j) = v;
+      }
+    } else if (EPI == EPI_RESIDUAL) {
+      // residual += sums; the next product's rows and this tile's share of the row's sum of squares
+      float* res = (float*)out + (int64_t)m * ldc;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int n = 16 * (tile_base + rt) + 4 * g4;
+        float ss = 0.f;
+        if (n < N) {
+          float v[4];
+          s16x4 p;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const bool in = n + i < N;
+            v[i] = in ? res[n + i] + acc[rt][mt][i] * scale[mt] : 0.f;
+            ss += v[i] * v[i];
+            p[i] = to_bf16_bits(in ? v[i] * load_param(norm.next_w, norm.next_w_is_f32, n + i) : 0.f);
+          }
+          bf16_t* nxt = norm.next_rows + (int64_t)m * norm.ld_next + n;
+          if (vec && norm.ld_next % 4 == 0 && n + 4 <= N) {
+            *reinterpret_cast<f32x4*>(res + n) = (f32x4){v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<s16x4*>(nxt) = p;
+          } else {
+            for (int i = 0; i < 4 && n + i < N; ++i) {
+              res[n + i] = v[i];
+              reinterpret_cast<short*>(nxt)[i] = p[i];
+            }
+          }
+        }
+        ss += __shfl_xor(ss, 16);  // the four lanes that hold this row's 16 columns
+        ss += __shfl_xor(ss, 32);
+        if (g4 == 0 && 16 * (tile_base + rt) < N) norm.next_stats[(int64_t)m * ((N + 15) / 16) + tile_base + rt] = ss;
       }
     } else {
 #pragma unroll
@@ -158,7 +256,7 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
         float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          v[i] = acc[rt][mt][i] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f);
+          v[i] = acc[rt][mt][i] * scale[mt] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f);
         if (EPI == EPI_F32) {
           float* dst = (float*)out + (int64_t)split * part_stride + (int64_t)m * ldc + n;
           if (vec && n + 4 <= N) *reinterpret_cast<f32x4*>(dst) = (f32x4){v[0], v[1], v[2], v[3]};
@@ -229,19 +327,26 @@ __device__ __forceinline__ bool add_up_k_ranges(f32x4 (&acc)[RT], int slot, int 
 // of a wavefront whose loads are in flight together.  With more
 // rows of A a workgroup takes more weight rows, so that the activations, which every
 // workgroup re-reads from L2, do not outweigh the weights.
-template <int MT, int RT, int EPI, int SKINNY_U>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out, int64_t ldc,
+template <int MT, int RT, int EPI, int SKINNY_U, int NW = 4>
+__global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__ out, int64_t ldc,
                                                           const bf16_t* __restrict__ A, int64_t lda,
                                                           const bf16_t* __restrict__ W,
                                                           const void* __restrict__ bias, int b_is_f32, int M,
                                                           int N, int K, int k_per_split, int64_t part_stride,
-                                                          SkinnyRope rope, SkinnyTickets tickets) {
-  __shared__ float s_part[MT == 1 ? 3 : 4][RT * MT * 4][PAE_WAVE];
+                                                          SkinnyRope rope, SkinnyTickets tickets, SkinnyNorm norm) {
+  static_assert(NW == 4 || MT == 1, "more than four wavefronts only with one column tile");
+  __shared__ float s_part[MT == 1 ? NW - 1 : 4][RT * MT * 4][PAE_WAVE];
   if (MT == 1 && gridDim.z > 1) {  // the rows of A are shared out in tiles of 16: this workgroup's tile
     const int m0 = blockIdx.z * 16;
     A += (int64_t)m0 * lda;
-    out = EPI == EPI_F32 ? (void*)((float*)out + (int64_t)m0 * ldc) : (void*)((bf16_t*)out + (int64_t)m0 * ldc);
+    out = (EPI == EPI_F32 || EPI == EPI_RESIDUAL) ? (void*)((float*)out + (int64_t)m0 * ldc)
+                                                  : (void*)((bf16_t*)out + (int64_t)m0 * ldc);
     M = min(16, M - m0);
+    if (norm.row_stats) norm.row_stats += (int64_t)m0 * norm.row_stat_tiles;
+    if (EPI == EPI_RESIDUAL) {
+      norm.next_rows += (int64_t)m0 * norm.ld_next;
+      norm.next_stats += (int64_t)m0 * ((N + 15) / 16);
+    }
     if (EPI == EPI_ROPE) {
       rope.positions += m0;
       if (rope.tok_seq) rope.tok_seq += m0;
@@ -250,6 +355,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
   }
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
+  float scale[MT];
   const int n0 = blockIdx.x * 16 * RT;
   const int k_lo = blockIdx.y * k_per_split;
   const int k_hi = min(K, k_lo + k_per_split);
@@ -287,13 +393,14 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
   // addresses, and issued SKINNY_U steps ahead of their use; a lane past the end of
   // the k range zeroes its weight fragment (rows past N or M are simply not stored).
   const bf16x8 zero = {};
-  struct Batch {  // SKINNY_U steps of a wavefront: k offsets kb + 128 u
+  constexpr int KW = 32 * NW;  // the workgroup's wavefronts take 32-wide k steps in turn
+  struct Batch {  // SKINNY_U steps of a wavefront: k offsets kb + KW u
     bf16x8 wf[SKINNY_U][RT], af[SKINNY_U][MT];
   };
   auto load = [&](Batch& b, int kb) {
 #pragma unroll
     for (int u = 0; u < SKINNY_U; ++u) {
-      const int k = kb + 128 * u + 8 * lkg;
+      const int k = kb + KW * u + 8 * lkg;
       const int kc = k < K - 8 ? k : K - 8;
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) b.wf[u][rt] = *reinterpret_cast<const bf16x8*>(wrow[rt] + kc);
@@ -305,7 +412,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
 #pragma unroll
     for (int u = 0; u < SKINNY_U; ++u) {
       // K and the range bounds are multiples of 8: a lane's 8 elements are all in or all out
-      const bool kok = kb + 128 * u + 8 * g4 < k_hi;
+      const bool kok = kb + KW * u + 8 * g4 < k_hi;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) b.af[u][mt] = to_mfma_order(b.af[u][mt], fetch_from);
 #pragma unroll
@@ -319,7 +426,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
       }
     }
   };
-  constexpr int STEP = 128 * SKINNY_U;
+  constexpr int STEP = KW * SKINNY_U;
   constexpr bool PIPELINED = true;
   int kb = k_lo + 32 * wave;  // the same in every lane of a wavefront: the branches on it are uniform
   if (PIPELINED) {
@@ -327,6 +434,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
     // batch waits out the memory's latency before the next is even asked for
     Batch b0, b1;
     if (kb < k_hi) load(b0, kb);
+    // asked for behind the first batch: loads come back in order, so the shares cost no wait of their own
+    row_scales<MT>(scale, norm, M, K);
     while (kb < k_hi) {
       if (kb + STEP < k_hi) load(b1, kb + STEP);
       multiply(b0, kb);
@@ -337,6 +446,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
       kb += STEP;
     }
   } else {  // more column tiles: the registers go to the activations' fragments
+    row_scales<MT>(scale, norm, M, K);
     for (; kb < k_hi; kb += STEP) {
       Batch b;
       load(b, kb);
@@ -356,7 +466,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
     __syncthreads();
     if (wave > 0) return;
 #pragma unroll
-    for (int w = 0; w < 3; ++w)
+    for (int w = 0; w < NW - 1; ++w)
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
@@ -400,7 +510,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ out
         for (int rt = 0; rt < RT; ++rt) acc[rt][mt] = mine[rt];
   }
   skinny_epilogue<MT, RT, EPI>(acc, blockIdx.x * RT, MT > 1 ? wave : -1, out, ldc, bias, b_is_f32, M, N, blockIdx.y,
-                               part_stride, rope);
+                               part_stride, rope, norm, scale);
 }
 
 // The same product for 17..64 rows of A where there are many weight rows.  With several column
@@ -417,11 +527,13 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
                                                           const bf16_t* __restrict__ W,
                                                           const void* __restrict__ bias, int b_is_f32, int M,
                                                           int N, int K, int k_per_split, int64_t part_stride,
-                                                          SkinnyRope rope, SkinnyTickets tickets) {
+                                                          SkinnyRope rope, SkinnyTickets tickets, SkinnyNorm norm) {
   constexpr int KC = 256 / RT, CH = KC / 128;
   __shared__ bf16x8 a_lds[2][MT][KC / 32][PAE_WAVE];  // [slab][column tile][k step][lane]
   const int tid = threadIdx.x, lane = tid % PAE_WAVE, wave = tid / PAE_WAVE;
   const int g4 = lane / 16;
+  float scale[MT];
+  row_scales<MT>(scale, norm, M, K);
   const int tile_base = (blockIdx.x * 4 + wave) * RT;  // this wavefront's first tile of 16 weight rows
   const int k_lo = blockIdx.y * k_per_split;
   const int k_hi = min(K, k_lo + k_per_split);
@@ -522,7 +634,7 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
                                   gridDim.y, tickets))
       return;
   }
-  skinny_epilogue<MT, RT, EPI>(acc, tile_base, -1, out, ldc, bias, b_is_f32, M, N, blockIdx.y, part_stride, rope);
+  skinny_epilogue<MT, RT, EPI>(acc, tile_base, -1, out, ldc, bias, b_is_f32, M, N, blockIdx.y, part_stride, rope, norm, scale);
 }
 
 // epilogue: 0 bfloat16 out (+bias), 1 float32 out (`splits` partials of `part_stride`
@@ -533,7 +645,7 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
 // sizes of the 1.5B, 7B and 72B models.
 static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
                          const void* bias, int b_is_f32, int M, int N, int K, int splits, int64_t part_stride,
-                         const SkinnyRope& rope, SkinnyTickets tickets, hipStream_t stream) {
+                         const SkinnyRope& rope, SkinnyTickets tickets, const SkinnyNorm& norm, hipStream_t stream) {
   PAE_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d is outside 0..64", M);
   PAE_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && lda % 8 == 0, "gemm_skinny: N=%d K=%d lda=%lld (K and lda must be multiples of 8)",
               N, K, (long long)lda);
@@ -542,6 +654,9 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
               "gemm_skinny: %d k ranges with epilogue %d need scratch for partial sums and tickets", splits, epilogue);
   PAE_REQUIRE(!(bias && splits > 1 && !ticketed), "gemm_skinny: a bias cannot be combined with partial sums");
   if (!ticketed) tickets = SkinnyTickets{nullptr, nullptr};
+  PAE_REQUIRE(!norm.row_stats || norm.row_stat_tiles > 0, "gemm_skinny: a row scale needs its shares of the sums of squares");
+  PAE_REQUIRE(epilogue != EPI_RESIDUAL || (norm.next_rows && norm.next_w && norm.next_stats && norm.ld_next >= N && !bias),
+              "gemm_skinny: the residual epilogue needs the next rows, the next norm's weight and room for its sums, and takes no bias");
   PAE_REQUIRE(epilogue != EPI_SWIGLU || (N % 16 == 0 && ldc % 4 == 0), "gemm_skinny: gated epilogue needs N %% 16 == 0, got %d", N);
   if (M == 0) return 0;
   // weight rows per workgroup: 16 for up to 16 rows of A, else 32 (see the kernel)
@@ -566,10 +681,10 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
 #define LAUNCH_MEDIUM(MT, EPI)                                                                                   \
   if (wide)                                                                                                      \
     gemm_medium_kernel<MT, 2, EPI><<<mgrid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W,  \
-                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets); \
+                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets, norm); \
   else                                                                                                           \
     gemm_medium_kernel<MT, 1, EPI><<<mgrid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W,  \
-                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets)
+                                                              bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets, norm)
 #define MEDIUM_BY_MT(EPI)                       \
   switch (mt) {                                 \
     case 2: LAUNCH_MEDIUM(2, EPI); break;       \
@@ -581,6 +696,7 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
       case EPI_F32: MEDIUM_BY_MT(EPI_F32); break;
       case EPI_SWIGLU: MEDIUM_BY_MT(EPI_SWIGLU); break;
       case EPI_ROPE: MEDIUM_BY_MT(EPI_ROPE); break;
+      case EPI_RESIDUAL: MEDIUM_BY_MT(EPI_RESIDUAL); break;
       default: return pae_fail("gemm_skinny: unknown epilogue %d", epilogue);
     }
 #undef MEDIUM_BY_MT
@@ -594,22 +710,31 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
     dim3 tiled((N + 15) / 16, splits, mt);
 #define LAUNCH_TILED(EPI)                                                                                        \
   gemm_skinny_kernel<1, 1, EPI, 4><<<tiled, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, bias, \
-                                                               b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets)
+                                                               b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets, norm)
     switch (epilogue) {
       case EPI_BF16: LAUNCH_TILED(EPI_BF16); break;
       case EPI_F32: LAUNCH_TILED(EPI_F32); break;
       case EPI_SWIGLU: LAUNCH_TILED(EPI_SWIGLU); break;
       case EPI_ROPE: LAUNCH_TILED(EPI_ROPE); break;
+      case EPI_RESIDUAL: LAUNCH_TILED(EPI_RESIDUAL); break;
       default: return pae_fail("gemm_skinny: unknown epilogue %d", epilogue);
     }
 #undef LAUNCH_TILED
     return pae_check_launch("gemm_skinny (rows of A in tiles)");
   }
+  if (epilogue == EPI_RESIDUAL && mt == 1 && splits == 1 && K >= 1024) {
+    // One k range, so that the sums are whole without tickets, and sixteen wavefronts to share it out:
+    // few workgroups, but each keeps its compute unit's memory pipeline full.
+    gemm_skinny_kernel<1, 1, EPI_RESIDUAL, 4, 16><<<dim3((N + 15) / 16, 1), 1024, 0, stream>>>(
+        out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, bias, b_is_f32, M, N, K, k_per_split, part_stride, rope,
+        tickets, norm);
+    return pae_check_launch("gemm_skinny (sixteen wavefronts)");
+  }
   dim3 grid((N + 16 * rt - 1) / (16 * rt), splits);
   // four k steps of loads in flight per wavefront: deeper prefetch costs registers and measured slower
 #define LAUNCH(MT, RT, EPI)                                                                                  \
   gemm_skinny_kernel<MT, RT, EPI, (MT == 1 ? 4 : 2)><<<grid, 256, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
-                                                               bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets)
+                                                               bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets, norm)
 #define BY_MT(EPI)                                                   \
   switch (mt) {                                                      \
     case 1: LAUNCH(1, 1, EPI); break;                                \
@@ -622,6 +747,7 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
     case EPI_F32: BY_MT(EPI_F32); break;
     case EPI_SWIGLU: BY_MT(EPI_SWIGLU); break;
     case EPI_ROPE: BY_MT(EPI_ROPE); break;
+    case EPI_RESIDUAL: BY_MT(EPI_RESIDUAL); break;
     default: return pae_fail("gemm_skinny: unknown epilogue %d", epilogue);
   }
 #undef BY_MT
@@ -629,16 +755,25 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   return pae_check_launch("gemm_skinny");
 }
 
+// row_stats (or null): the rows of A are bfloat16(x * w_norm) of a row x that is still to be divided
+// by its root mean square; row_stats[m][0 .. row_stat_tiles) add up to sum(x^2) and the sums of row m
+// are multiplied by rsqrt(that / K + row_eps).  Epilogue 4 adds the sums into the float32 `out`
+// (the residual) in place and leaves bfloat16(out * next_w) in next_rows and the shares of the new
+// rows' sums of squares in next_stats[M][(N + 15) / 16].
 // Several k ranges with an epilogue other than float32 partial sums are added up inside the kernel:
 // ticket_parts is scratch of pae_skinny_ticket_floats(M, N, splits) floats and ticket_counters holds
 // pae_skinny_ticket_slots(M, N) ints that are zero before the call and zero after it.  Launches that
 // share the counters must not overlap.
 extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
                                const void* bias, int b_is_f32, int M, int N, int K, int splits,
-                               int64_t part_stride, float* ticket_parts, int* ticket_counters, hipStream_t stream) {
+                               int64_t part_stride, float* ticket_parts, int* ticket_counters,
+                               const float* row_stats, int row_stat_tiles, float row_eps, void* next_rows,
+                               int64_t ld_next, const void* next_w, int next_w_is_f32, float* next_stats,
+                               hipStream_t stream) {
   PAE_REQUIRE(epilogue != EPI_ROPE, "gemm_skinny: the rotating epilogue has an entry point of its own");
+  const SkinnyNorm norm{row_stats, row_stat_tiles, row_eps, (bf16_t*)next_rows, ld_next, next_w, next_w_is_f32, next_stats};
   return launch_skinny(epilogue, out, ldc, A, lda, W, bias, b_is_f32, M, N, K, splits, part_stride, SkinnyRope{},
-                       SkinnyTickets{ticket_parts, ticket_counters}, stream);
+                       SkinnyTickets{ticket_parts, ticket_counters}, norm, stream);
 }
 
 // Counters and scratch floats that `splits` k ranges of an [M, K] x [N, K]^T product need for their
@@ -658,7 +793,8 @@ extern "C" int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int
                                     const void* bias, int b_is_f32, int M, int K, int nh, int nkv, int hd, int rot,
                                     const float* cos_sin, const int* positions, const int* tok_seq,
                                     const int* block_tables, int max_blocks, int bs, void* k_cache, void* v_cache,
-                                    int splits, float* ticket_parts, int* ticket_counters, hipStream_t stream) {
+                                    int splits, float* ticket_parts, int* ticket_counters, const float* row_stats,
+                                    int row_stat_tiles, float row_eps, hipStream_t stream) {
   PAE_REQUIRE(nh > 0 && nkv >= 0 && hd > 0 && hd % 16 == 0, "gemm_skinny_rope: bad head sizes nh=%d nkv=%d hd=%d", nh, nkv, hd);
   PAE_REQUIRE(rot >= 0 && rot <= hd && rot % 16 == 0 && (rot == 0 || cos_sin),
               "gemm_skinny_rope: rotary_dim %d must be a multiple of 16 up to head_dim %d", rot, hd);
@@ -668,6 +804,7 @@ extern "C" int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int
               "gemm_skinny_rope: the cache write needs tables and pools");
   SkinnyRope rope{cos_sin, positions, tok_seq, block_tables, (bf16_t*)k_cache, (bf16_t*)v_cache,
                   nh, nkv, hd, rot, max_blocks, bs};
+  const SkinnyNorm norm{row_stats, row_stat_tiles, row_eps, nullptr, 0, nullptr, 0, nullptr};
   return launch_skinny(EPI_ROPE, q_out, ldq, A, lda, W, bias, b_is_f32, M, (nh + 2 * nkv) * hd, K, splits, 0, rope,
-                       SkinnyTickets{ticket_parts, ticket_counters}, stream);
+                       SkinnyTickets{ticket_parts, ticket_counters}, norm, stream);
 }

@@ -20,7 +20,7 @@ from ..cache.manager import CacheManager, bytes_of_one_page_everywhere
 from ..config.model_config import ModelPlan
 from ..config.registry import read_config, read_config_dict
 from ..kernels import lib as K
-from ..parts import ResidualStream, StepContext, build_block, build_part
+from ..parts import OwedRows, ResidualStream, StepContext, build_block, build_part
 from ..parts.base import NORMS
 from ..parts.linear import Linear
 from ..weights.loader import load_weights
@@ -129,13 +129,28 @@ class Model:
         [len(logit_rows), vocab] at the flat rows `logit_rows` (int32)."""
         self.forward_pass_count += 1
         plan = self.plan
-        residual = torch.empty((ctx.num_tokens, plan.hidden_size), dtype=torch.float32, device=self.device)
-        K.embedding(residual, self.embedding, token_ids, plan.embedding_scale)
+        T, H = ctx.num_tokens, plan.hidden_size
+        residual = torch.empty((T, H), dtype=torch.float32, device=self.device)
         stream = ResidualStream(residual)
+        # the norm that reads the stream first at every stop (and the final norm after the last)
+        first_norms = [getattr(self.blocks[entry.layer], "mixer_norm", None) for entry in plan.schedule] + [self.final_norm]
+        fold = getattr(first_norms[0], "folded", None)
+        first_mixer = getattr(self.blocks[plan.schedule[0].layer], "mixer", None) if plan.schedule else None
+        if (self.dtype == torch.bfloat16 and fold is not None and 0 < T <= K.FOLD_MAX_ROWS and H % 8 == 0
+                and getattr(first_mixer, "takes_owed_rows", False)):
+            # few rows: the first norm is paid by the first product (see parts.OwedRows)
+            weight, eps = fold()
+            rows = torch.empty((T, H), dtype=torch.bfloat16, device=self.device)
+            stats = torch.empty((T, K.stat_tiles(H)), dtype=torch.float32, device=self.device)
+            K.embedding_rows(residual, self.embedding, token_ids, plan.embedding_scale, rows, weight, stats)
+            stream.owed, stream.owed_to = OwedRows(rows, stats, eps), first_norms[0]
+        else:
+            K.embedding(residual, self.embedding, token_ids, plan.embedding_scale)
         for index, entry in enumerate(plan.schedule):
             ctx.entry = index
             ctx.cache_entry = index if entry.cache_from is None else entry.cache_from
             ctx.writes_cache = entry.cache_from is None
+            stream.next_norm = first_norms[index + 1]
             self.blocks[entry.layer].forward(ctx, stream)
         rows = logit_rows.numel()
         if rows == 0:

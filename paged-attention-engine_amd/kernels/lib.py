@@ -59,8 +59,10 @@ def _declare(lib) -> None:
         "pae_rope_table": [P, P, P, I, I, P],
         "pae_rope_kv_write": [I, P, L, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P],
         "pae_swiglu": [I, P, P, I, I, I, P],
-        "pae_gemm_skinny": [I, P, L, P, L, P, P, I, I, I, I, I, L, P, P, P],
-        "pae_gemm_skinny_rope": [P, L, P, L, P, P, I, I, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P, P, P],
+        "pae_gemm_skinny": [I, P, L, P, L, P, P, I, I, I, I, I, L, P, P, P, I, F, P, L, P, I, P, P],
+        "pae_gemm_skinny_rope": [P, L, P, L, P, P, I, I, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P, P, P, I, F, P],
+        "pae_embedding_rows": [I, P, P, P, I, I, I, F, P, P, I, P, P],
+        "pae_scaled_rows": [P, P, P, I, F, I, I, P],
         "pae_skinny_ticket_slots": [I, I],
         "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
@@ -259,7 +261,54 @@ def swiglu(out: torch.Tensor, x: torch.Tensor, block: int = 0) -> None:
 
 
 SKINNY_MAX_ROWS = 64
-EPI_BF16, EPI_F32, EPI_SWIGLU = 0, 1, 2
+FOLD_MAX_ROWS = 16  # up to this many rows a norm is folded into the products around it (see parts.OwedRows)
+EPI_BF16, EPI_F32, EPI_SWIGLU, EPI_RESIDUAL = 0, 1, 2, 4
+
+
+def stat_tiles(width: int) -> int:
+    """Shares a row's sum of squares is kept in: one per 16 columns."""
+    return -(-width // 16)
+
+
+def _row_scale(row_scale, M: int, K: int):
+    """(pointer, tiles, eps) of the shares of the rows' sums of squares, for a product whose rows
+    are still to be divided by their root mean square; (None, 0, 0) for plain rows."""
+    if row_scale is None:
+        return None, 0, 0.0
+    stats, eps = row_scale
+    assert stats.is_cuda and stats.dtype == torch.float32 and stats.is_contiguous()
+    assert stats.dim() == 2 and stats.shape[0] >= M and stats.shape[1] == stat_tiles(K)
+    return stats.data_ptr(), stats.shape[1], float(eps)
+
+
+def embedding_rows(residual: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float,
+                   next_rows: torch.Tensor, next_w: torch.Tensor, next_stats: torch.Tensor) -> None:
+    """`embedding` for a step whose first norm is folded into the products: beside residual[t] =
+    scale * table[ids[t]], next_rows[t] = bfloat16(residual[t] * next_w) and next_stats[t][j] = the sum
+    of squares of residual[t] over columns 16 j .. 16 j + 15."""
+    _gpu(residual, table, ids, next_rows, next_w, next_stats)
+    T, H = residual.shape
+    assert residual.dtype == torch.float32 and residual.is_contiguous() and table.is_contiguous()
+    assert ids.dtype == torch.int32 and ids.numel() == T and table.shape[1] == H
+    assert next_rows.dtype == torch.bfloat16 and next_rows.shape == (T, H) and next_rows.is_contiguous()
+    assert next_stats.dtype == torch.float32 and next_stats.shape == (T, stat_tiles(H)) and next_stats.is_contiguous()
+    assert next_w.numel() == H
+    wp, wf = _param(next_w)
+    _check(library().pae_embedding_rows(code_of(table.dtype), residual.data_ptr(), table.data_ptr(), ids.data_ptr(),
+                                        T, H, table.shape[0], float(scale), next_rows.data_ptr(), wp, wf,
+                                        next_stats.data_ptr(), _stream()))
+
+
+def scaled_rows(rows: torch.Tensor, stats: torch.Tensor, eps: float) -> torch.Tensor:
+    """rows[m] * rsqrt(sum(stats[m]) / width + eps) as bfloat16: rows whose scale was owed, paid."""
+    _gpu(rows, stats)
+    M, H = rows.shape
+    assert rows.dtype == torch.bfloat16 and rows.is_contiguous()
+    assert stats.dtype == torch.float32 and stats.shape == (M, stat_tiles(H)) and stats.is_contiguous()
+    out = torch.empty_like(rows)
+    _check(library().pae_scaled_rows(out.data_ptr(), rows.data_ptr(), stats.data_ptr(), stats.shape[1], float(eps),
+                                     M, H, _stream()))
+    return out
 
 
 def skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -297,29 +346,48 @@ def skinny_splits(N: int, K: int, M: int = 1) -> int:
 
 
 def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
-                epilogue: int = EPI_BF16, splits: int = 1) -> None:
+                epilogue: int = EPI_BF16, splits: int = 1, row_scale=None, following=None) -> None:
     """out = a @ w^T for at most 64 rows of `a`, reading `w` once.
 
     EPI_BF16: out [M, N] bfloat16 (+bias).  EPI_F32: out [M, N] float32, or [splits, M, N]
     partial sums over k ranges.  EPI_SWIGLU: w holds blocks of 8 gate rows followed by their 8
     up rows; out [M, N / 2] = silu(gate) * up.  With several k ranges the other epilogues'
-    partial sums are added up inside the kernel (see `skinny_tickets`)."""
+    partial sums are added up inside the kernel (see `skinny_tickets`).
+
+    `row_scale = (stats, eps)`: the rows of `a` are bfloat16(x * w_norm) of rows x that are still
+    to be divided by their root mean square; `stats[m]` holds shares that add up to sum(x[m]^2),
+    and row m's sums are multiplied by rsqrt(that / K + eps) before the epilogue.
+    EPI_RESIDUAL: `out` is the float32 residual [M, N], to which the product is added in place;
+    `following = (next_rows, next_w, next_stats)` receives bfloat16(out * next_w) [M, N] and the
+    shares [M, stat_tiles(N)] of the new rows' sums of squares, for the product after the next norm."""
     _gpu(out, a, w, bias)
     M, K_ = a.shape
     N = w.shape[0]
     assert skinny_supported(a, w) and w.shape == (N, K_) and w.is_contiguous() and out.is_contiguous()
+    nr = nw = ns = None
+    nwf, ld_next = 0, 0
     if epilogue == EPI_SWIGLU:
         assert out.shape == (M, N // 2) and out.dtype == torch.bfloat16 and bias is None
     elif epilogue == EPI_F32:
         assert out.dtype == torch.float32
         assert tuple(out.shape) == ((M, N) if splits == 1 and out.dim() == 2 else (splits, M, N))
+    elif epilogue == EPI_RESIDUAL:
+        assert out.shape == (M, N) and out.dtype == torch.float32 and bias is None and following is not None
+        next_rows, next_w, next_stats = following
+        _gpu(next_rows, next_w, next_stats)
+        assert next_rows.dtype == torch.bfloat16 and next_rows.shape == (M, N) and next_rows.stride(1) == 1
+        assert next_stats.dtype == torch.float32 and next_stats.shape == (M, stat_tiles(N)) and next_stats.is_contiguous()
+        assert next_w.numel() == N
+        nr, ns, ld_next = next_rows.data_ptr(), next_stats.data_ptr(), next_rows.stride(0)
+        nw, nwf = _param(next_w)
     else:
         assert out.shape == (M, N) and out.dtype == torch.bfloat16
     bp, bf = _param(bias)
+    sp, st, se = _row_scale(row_scale, M, K_)
     parts, counters = _ticket_scratch(a.device, M, N, splits if epilogue != EPI_F32 else 1)
     _check(library().pae_gemm_skinny(epilogue, out.data_ptr(), out.stride(-2), a.data_ptr(), a.stride(0),
                                      w.data_ptr(), bp, bf, M, N, K_, splits, M * N, _ptr(parts), _ptr(counters),
-                                     _stream()))
+                                     sp, st, se, nr, ld_next, nw, nwf, ns, _stream()))
 
 
 _TICKETS: dict = {}
@@ -380,7 +448,7 @@ def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias
                      nkv: int, hd: int, rot: int, cos_sin: Optional[torch.Tensor], positions: torch.Tensor,
                      tok_seq: Optional[torch.Tensor], block_tables: Optional[torch.Tensor], block_size: int,
                      k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                     splits: Optional[int] = None) -> None:
+                     splits: Optional[int] = None, row_scale=None) -> None:
     """Query/key/value projection of at most 64 rows with the rotation and the cache write in its
     epilogue: q_out[M, nh * hd] = rotated queries; rotated keys and raw values go to their slots
     (nkv == 0: `w` holds the query rows only and nothing is stored).  `cos_sin`: see `rope_table`."""
@@ -401,11 +469,12 @@ def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias
     lib, N = library(), w.shape[0]
     splits = 1 if splits is None else splits
     parts, counters = _ticket_scratch(a.device, M, N, splits)
+    sp, st, se = _row_scale(row_scale, M, K_)
     _check(lib.pae_gemm_skinny_rope(q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(),
                                     bp, bf, M, K_, nh, nkv, hd, rot, _ptr(cos_sin) if rot else None,
                                     positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks,
                                     block_size, _ptr(k_cache), _ptr(v_cache), splits, _ptr(parts), _ptr(counters),
-                                    _stream()))
+                                    sp, st, se, _stream()))
 
 
 def gemm_plain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:

@@ -24,7 +24,7 @@ import torch
 
 from ..cache.manager import attention_pages
 from ..kernels import lib as K
-from .base import POSITION_ENCODINGS, Part, StepShape, build_part, register_mixer
+from .base import POSITION_ENCODINGS, OwedRows, Part, StepShape, build_part, plain_rows, register_mixer
 from .linear import Linear, rows_a_graph_may_hold
 
 WORK_LISTS = ("paged attention work lists", K.PREFILL_TILE)
@@ -48,6 +48,8 @@ def attention_work_lists(shape: StepShape):
 
 @register_mixer("attention")
 class PagedAttention(Part):
+    takes_owed_rows = True
+
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         if spec.num_heads % spec.num_kv_heads:
@@ -115,9 +117,12 @@ class PagedAttention(Part):
         else:
             linear, nkv, k_cache, v_cache, table = self.q_only, 0, None, None, None
         rotary = getattr(self.position, "rotary_table", None)
+        owed = x if isinstance(x, OwedRows) else None
+        if owed is not None:
+            x = owed.rows
         if rotary is None:
             # any encoding: project, let it encode query and key heads in place, then store
-            qkv = linear(x)
+            qkv = linear(owed if owed is not None else x)
             self.position.encode(ctx, qkv, s.num_heads + nkv, s.head_dim)
             if nkv:
                 K.kv_store(qkv, s.num_heads, nkv, s.head_dim, ctx.positions, ctx.tok_seq, table, bs, k_cache, v_cache)
@@ -128,14 +133,16 @@ class PagedAttention(Part):
             q = torch.empty((x.shape[0], s.num_heads * s.head_dim), dtype=x.dtype, device=x.device)
             splits = K.whole_sum_splits(linear.out_features, linear.in_features, x.shape[0])
             K.gemm_skinny_rope(q, x, linear.weight, linear.bias, s.num_heads, nkv, s.head_dim, rot, cos_sin,
-                               ctx.positions, ctx.tok_seq, table, bs, k_cache, v_cache, splits)
+                               ctx.positions, ctx.tok_seq, table, bs, k_cache, v_cache, splits,
+                               row_scale=owed.row_scale if owed is not None else None)
             return q
-        qkv = linear(x)
+        qkv = linear(owed if owed is not None else x)
         K.rope_kv_write(qkv, s.num_heads, nkv, s.head_dim, rot, cos_sin, ctx.positions, ctx.tok_seq, table, bs,
                         k_cache, v_cache)
         return qkv
 
-    def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, ctx, x):
+        """`x`: normalised activations, or `OwedRows` (the projection then pays their scale)."""
         s = self.spec
         k_cache, v_cache = ctx.cache.kv_of(ctx.cache_entry)
         table = ctx.block_tables[ctx.cache.group_of(ctx.cache_entry)]
@@ -151,4 +158,4 @@ class PagedAttention(Part):
                 K.attn_prefill(attn, qkv, k_cache, v_cache, prefill_tiles, ctx.positions, table, *geometry)
         else:
             K.paged_attention_generic(attn, qkv, k_cache, v_cache, ctx.positions, ctx.tok_seq, table, *geometry)
-        return self.out.branch(attn)
+        return self.out.branch(attn, ctx.sink)

@@ -24,15 +24,75 @@ from typing import Callable, Dict, List, Mapping, Optional, Tuple
 import torch
 
 
+class OwedRows:
+    """Activations whose division by their root mean square is still owed.
+
+    `rows` = bfloat16(x * w) for the input x and the weight w of a norm; `stats[m]` holds shares
+    that add up to sum(x[m]^2) (one per 16 columns).  norm(x) W^T = rsqrt(mean(x^2) + eps) *
+    (rows W^T), so a matrix product can pay the scale on its finished sums, and a decode step
+    needs no norm kernel between its products.  A part that wants plain activations calls
+    `settle()`."""
+
+    def __init__(self, rows: torch.Tensor, stats: torch.Tensor, eps: float) -> None:
+        self.rows, self.stats, self.eps = rows, stats, eps
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    @property
+    def dtype(self):
+        return self.rows.dtype
+
+    @property
+    def device(self):
+        return self.rows.device
+
+    @property
+    def row_scale(self):
+        return self.stats, self.eps
+
+    def settle(self) -> torch.Tensor:
+        from ..kernels import lib as K
+        return K.scaled_rows(self.rows, self.stats, self.eps)
+
+
+def plain_rows(x):
+    """`x` as plain activations, whatever form it came in."""
+    return x.settle() if isinstance(x, OwedRows) else x
+
+
 class ResidualStream:
     """The float32 residual sum of a step and the branch output not yet added to it.
 
     Norm parts add `pending` while they normalise, so the sum is formed in
-    32-bit and written once."""
+    32-bit and written once.  A branch whose last product can add itself into the residual
+    (see `BranchSink`) leaves no `pending` but `owed`, the rows prepared for the norm `owed_to`."""
 
     def __init__(self, residual: torch.Tensor) -> None:
         self.residual = residual
         self.pending: Optional[torch.Tensor] = None
+        self.owed: Optional[OwedRows] = None
+        self.owed_to: Optional[object] = None
+        self.next_norm: Optional[object] = None  # set by the model: the norm that reads the stream after this block
+
+
+class BranchSink:
+    """Where a branch's last product may deliver itself instead of returning its output: added
+    into the stream's residual in place, with the rows the following norm's consumer wants
+    prepared on the way.  `norm` is the norm part that will read the stream next; it must offer
+    `folded() -> (weight, eps)` for the offer to be taken up."""
+
+    def __init__(self, stream: ResidualStream, norm) -> None:
+        self.stream, self.norm = stream, norm
+
+    def folded(self):
+        fold = getattr(self.norm, "folded", None)
+        return fold() if fold is not None else None
+
+    def deliver(self, owed: OwedRows) -> None:
+        self.stream.pending = None
+        self.stream.owed, self.stream.owed_to = owed, self.norm
 
 
 @dataclass(frozen=True)
@@ -75,6 +135,7 @@ class StepContext:
     entry: int = 0                     # index in the schedule
     cache_entry: int = 0               # the stop whose cache is read (entry itself unless it borrows)
     writes_cache: bool = True
+    sink: Optional["BranchSink"] = None  # set by the block around a branch: see BranchSink
     # what a part computes once per step for every layer that has the same part (a table of angles,
     # say), under a key of the part's choosing; the step function also leaves here, under
     # `step_lists_key`, the index lists a part asked for (`Part.step_lists`), as int32 device tensors
@@ -91,6 +152,9 @@ class Part:
     # The most rows of a step for which that holds (None: any number): a part whose products
     # leave this engine's kernels above some row count says so here.
     graph_max_rows: Optional[int] = None
+    # True when `forward` takes its input as `OwedRows` as well as a plain tensor (the block
+    # settles them for parts that do not).
+    takes_owed_rows = False
 
     def __init__(self, spec, dtype: torch.dtype, device) -> None:
         self.spec = spec

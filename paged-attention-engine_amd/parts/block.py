@@ -7,7 +7,8 @@ left pending on the stream and added by the next norm, in float32.
 
 from __future__ import annotations
 
-from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Part, ResidualStream, build_part, register_block)
+from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BranchSink, Part, ResidualStream, build_part, plain_rows,
+                   register_block)
 
 
 @register_block("prenorm")
@@ -49,10 +50,16 @@ class PreNormBlock:
             part.bind(prefix, weights)
 
     def forward(self, ctx, stream: ResidualStream) -> None:
+        """Each branch is offered a sink: its last product may add itself into the residual and
+        prepare the rows of the norm that reads the stream next (this block's second norm, then
+        `stream.next_norm`, the first norm of the block that follows), which then runs no kernel."""
         x = self.mixer_norm.forward(stream)
-        stream.pending = self.mixer.forward(ctx, x)
+        ctx.sink = BranchSink(stream, self.feed_forward_norm)
+        stream.pending = self.mixer.forward(ctx, x if self.mixer.takes_owed_rows else plain_rows(x))
         x = self.feed_forward_norm.forward(stream)
-        stream.pending = self.feed_forward.forward(ctx, x)
+        ctx.sink = BranchSink(stream, stream.next_norm) if stream.next_norm is not None else None
+        stream.pending = self.feed_forward.forward(ctx, x if self.feed_forward.takes_owed_rows else plain_rows(x))
+        ctx.sink = None
 
 
 def build_block(layer_spec, dtype, device):

@@ -19,6 +19,7 @@ from typing import Optional
 import torch
 
 from ..kernels import lib as K
+from .base import OwedRows
 
 
 def rows_a_graph_may_hold(dtype: torch.dtype, *inner_sizes: int):
@@ -50,8 +51,14 @@ class Linear:
             torch.addmm(bias if bias.dtype == x.dtype else bias.to(x.dtype), x, self.weight.t(), out=out)
         return out
 
-    def __call__(self, x: torch.Tensor) -> torch.Tensor:
-        """[M, N] in x's dtype."""
+    def __call__(self, x) -> torch.Tensor:
+        """[M, N] in x's dtype.  `x` may be `OwedRows`: the few-row product pays their scale itself."""
+        if isinstance(x, OwedRows):
+            if x.shape[0] and K.skinny_supported(x.rows, self.weight):
+                out = torch.empty((x.shape[0], self.out_features), dtype=x.dtype, device=x.device)
+                K.gemm_skinny(out, x.rows, self.weight, self.bias, K.EPI_BF16, row_scale=x.row_scale)
+                return out
+            x = x.settle()
         M = x.shape[0]
         if x.dtype == torch.float32 or M == 0:
             out = torch.empty((M, self.out_features), dtype=x.dtype, device=x.device)
@@ -64,11 +71,23 @@ class Linear:
             return out
         return self._library(x)
 
-    def branch(self, x: torch.Tensor) -> torch.Tensor:
+    def branch(self, x: torch.Tensor, sink=None) -> Optional[torch.Tensor]:
         """The product as a residual branch's output: [M, N] in x's dtype, or float32
-        partial sums [P, M, N] that the next norm adds up in order (no bias then)."""
+        partial sums [P, M, N] that the next norm adds up in order (no bias then).  With a `sink`
+        whose norm can be folded, the few-row product adds itself into the residual instead and
+        prepares the following product's rows; nothing is returned then."""
         if x.dtype == torch.bfloat16 and self.bias is None and x.shape[0] and K.skinny_supported(x, self.weight):
             splits = K.skinny_splits(self.out_features, self.in_features, x.shape[0])
+            fold = sink.folded() if sink is not None else None
+            residual = sink.stream.residual if sink is not None else None
+            if (fold is not None and x.shape[0] <= K.FOLD_MAX_ROWS and residual.dtype == torch.float32
+                    and residual.is_contiguous() and tuple(residual.shape) == (x.shape[0], self.out_features)):
+                weight, eps = fold
+                rows = torch.empty((x.shape[0], self.out_features), dtype=torch.bfloat16, device=x.device)
+                stats = torch.empty((x.shape[0], K.stat_tiles(self.out_features)), dtype=torch.float32, device=x.device)
+                K.gemm_skinny(residual, x, self.weight, None, K.EPI_RESIDUAL, splits, following=(rows, weight, stats))
+                sink.deliver(OwedRows(rows, stats, eps))
+                return None
             out = torch.empty((splits, x.shape[0], self.out_features), dtype=torch.float32, device=x.device)
             K.gemm_skinny(out, x, self.weight, None, K.EPI_F32, splits)
             return out

@@ -7,13 +7,14 @@ from __future__ import annotations
 import torch
 
 from ..kernels import lib as K
-from .base import Part, register_feed_forward
+from .base import OwedRows, Part, plain_rows, register_feed_forward
 from .linear import Linear, rows_a_graph_may_hold
 
 
 @register_feed_forward("swiglu")
 class SwiGLU(Part):
     graph_safe = True
+    takes_owed_rows = True
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         if spec.activation != "silu":
@@ -44,11 +45,14 @@ class SwiGLU(Part):
         self.gate_up = Linear(self.matrix(gate_up))
         self.down = Linear(self.matrix(weights[prefix + "down_proj.weight"]))
 
-    def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, ctx, x):
+        """`x`: normalised activations, or `OwedRows` (the gated product then pays their scale)."""
         act = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
-        if self.block and x.shape[0] and K.skinny_supported(x, self.gate_up.weight):
+        rows = x.rows if isinstance(x, OwedRows) else x
+        if self.block and x.shape[0] and K.skinny_supported(rows, self.gate_up.weight):
             splits = K.whole_sum_splits(2 * self.spec.intermediate_size, self.spec.hidden_size, x.shape[0])
-            K.gemm_skinny(act, x, self.gate_up.weight, None, K.EPI_SWIGLU, splits)
+            K.gemm_skinny(act, rows, self.gate_up.weight, None, K.EPI_SWIGLU, splits,
+                          row_scale=x.row_scale if isinstance(x, OwedRows) else None)
         else:
-            K.swiglu(act, self.gate_up(x), self.block)
-        return self.down.branch(act)
+            K.swiglu(act, self.gate_up(plain_rows(x)), self.block)
+        return self.down.branch(act, getattr(ctx, "sink", None))

@@ -116,6 +116,75 @@ def test_gemm_skinny(M, N, K_):
         assert torch.equal(one[0], out32[M - 1])
 
 
+@pytest.mark.parametrize("M", [1, 8, 17, 40, 64])
+@pytest.mark.parametrize("N,K_,ranges", [(1536, 1536, 4), (1536, 8960, 5), (200, 72, 1), (72, 200, 1), (3584, 512, 2),
+                                          (8192, 1024, 3)])
+def test_a_norm_folded_into_the_products_around_it(M, N, K_, ranges):
+    """The product that ends a branch adds itself into the float32 residual and leaves, for the
+    product after the next norm, the rows bfloat16(residual * w_norm) and the shares of every
+    row's sum of squares; that product multiplies its sums by rsqrt(mean square + eps).  Together
+    they give what add + RMSNorm + product give, without a norm kernel in between."""
+    torch.manual_seed(M * 7 + N)
+    eps = 1e-5
+    a = (torch.randn(M, K_) * 0.5).to(torch.bfloat16)
+    w = (torch.randn(N, K_) * 0.1).to(torch.bfloat16)
+    residual = torch.randn(M, N) * 2.0
+    w_norm = (1 + 0.2 * torch.randn(N)).to(torch.bfloat16)
+    want_residual = residual.double() + a.double() @ w.double().t()
+    res_d = residual.to(DEV)
+    next_rows = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    stats = torch.full((M, K().stat_tiles(N)), float("nan"), dtype=torch.float32, device=DEV)
+    K().gemm_skinny(res_d, a.to(DEV), w.to(DEV), None, K().EPI_RESIDUAL, ranges,
+                    following=(next_rows, w_norm.to(DEV), stats))
+    top = float(want_residual.abs().max())
+    assert (res_d.double().cpu() - want_residual).abs().max() <= 2e-5 * top
+    want_rows = (res_d.cpu() * w_norm.float()).to(torch.bfloat16)
+    assert (next_rows.float().cpu() - want_rows.float()).abs().max() <= 2.0 ** -7 * float(want_rows.float().abs().max())
+    assert torch.allclose(stats.sum(1).double().cpu(), res_d.double().cpu().pow(2).sum(1), rtol=1e-5)
+    # the same again lands on top of the first (the residual is updated in place)
+    K().gemm_skinny(res_d, a.to(DEV), w.to(DEV), None, K().EPI_RESIDUAL, 1, following=(next_rows, w_norm.to(DEV), stats))
+    want2 = want_residual + a.double() @ w.double().t()
+    assert (res_d.double().cpu() - want2).abs().max() <= 4e-5 * float(want2.abs().max())
+
+    # the consumer: a product over the rows whose scale is owed, against norm-then-product
+    x = res_d.double().cpu()
+    normed = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w_norm.double()
+    if N % 8:
+        return  # the consumer's inner size must be a multiple of 8
+    for N2 in (48, 1000):
+        w2 = (torch.randn(N2, N) * 0.1).to(torch.bfloat16)
+        b2 = torch.randn(N2).to(torch.bfloat16)
+        want = normed @ w2.double().t() + b2.double()
+        out = torch.empty(M, N2, dtype=torch.bfloat16, device=DEV)
+        K().gemm_skinny(out, next_rows, w2.to(DEV), b2.to(DEV), K().EPI_BF16, row_scale=(stats, eps))
+        assert (out.double().cpu() - want).abs().max() <= 2.0 ** -6 * (float(want.abs().max()) + 1)
+        splits = 2 if N >= 1024 else 1
+        out2 = torch.empty(M, N2, dtype=torch.bfloat16, device=DEV)
+        K().gemm_skinny(out2, next_rows, w2.to(DEV), b2.to(DEV), K().EPI_BF16, splits, row_scale=(stats, eps))
+        assert (out2.double().cpu() - want).abs().max() <= 2.0 ** -6 * (float(want.abs().max()) + 1)
+    # rows whose scale is paid by a kernel of its own, for parts that want plain activations
+    plain_rows = K().scaled_rows(next_rows, stats, eps)
+    assert (plain_rows.double().cpu() - normed).abs().max() <= 2.0 ** -6 * float(normed.abs().max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embedding_rows(dtype):
+    torch.manual_seed(3)
+    V, H, T = 333, 200, 9
+    table = torch.randn(V, H).to(DT[dtype])
+    ids = torch.randint(0, V, (T,), dtype=torch.int32)
+    w_norm = (1 + 0.1 * torch.randn(H)).to(torch.bfloat16)
+    residual = torch.empty(T, H, dtype=torch.float32, device=DEV)
+    rows = torch.empty(T, H, dtype=torch.bfloat16, device=DEV)
+    stats = torch.empty(T, K().stat_tiles(H), dtype=torch.float32, device=DEV)
+    K().embedding_rows(residual, table.to(DEV), ids.to(DEV), 1.5, rows, w_norm.to(DEV), stats)
+    want = 1.5 * table[ids.long()].float()
+    assert torch.equal(residual.cpu(), want)
+    assert torch.equal(rows.cpu(), (want * w_norm.float()).to(torch.bfloat16))
+    assert torch.allclose(stats.sum(1).cpu(), want.pow(2).sum(1), rtol=1e-5)
+    assert torch.allclose(stats[:, -1].cpu(), want[:, 192:].pow(2).sum(1), rtol=1e-5)  # the last, short tile
+
+
 @pytest.mark.parametrize("M", [17, 40, 64])
 @pytest.mark.parametrize("N,K_", [(32777, 264), (9000, 1024), (151936, 72)])
 def test_gemm_many_weight_rows(M, N, K_):
