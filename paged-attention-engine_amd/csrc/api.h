@@ -49,9 +49,9 @@ int pae_paged_attention_generic(int dtype, void* out, int64_t out_stride, const 
                                 hipStream_t stream);
 int pae_attn_decode_split();
 int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
-                         const void* v_cache, const int* dec_tok, int num_dec, const int* positions,
-                         const int* tok_seq, const int* block_tables, int max_blocks, int bs, int nh, int nkv,
-                         int hd, float scale, int window, void* part_acc, void* part_ml, hipStream_t stream);
+                         const void* v_cache, const int* dec_work, int num_dec, const int* block_tables,
+                         int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window, void* part_acc,
+                         void* part_ml, hipStream_t stream);
 int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
                           const void* v_cache, const int* tiles, int num_tiles, const int* positions,
                           const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,

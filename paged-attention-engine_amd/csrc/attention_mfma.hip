@@ -137,19 +137,21 @@ template <int HD, int TPW>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     float* __restrict__ part_acc, float* __restrict__ part_ml, int max_splits,
     const bf16_t* __restrict__ q, int64_t q_stride,
-    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ dec_tok,
-    const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_tables,
-    int max_blocks, int bs, int nh, int nkv, float scale_log2, int window) {
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int4* __restrict__ dec_work,
+    const int* __restrict__ block_tables, int max_blocks, int bs, int nh, int nkv, float scale_log2, int window) {
   constexpr int SPLIT = 64 * TPW;
   const int split = blockIdx.x, kvh = blockIdx.y;
-  const int tok = dec_tok[blockIdx.z];
-  const int pos[1] = {positions[tok]};
+  // one load brings the token's row, its position and its table row: a chain of three dependent
+  // loads (token, then position and sequence, then pages) would cost a trip to memory each
+  const int4 work = dec_work[blockIdx.z];
+  const int tok = work.x;
+  const int pos[1] = {work.y};
   const int start[1] = {(window > 0 && pos[0] - window + 1 > 0) ? pos[0] - window + 1 : 0};
   const int s_first = start[0] / SPLIT, s_last = pos[0] / SPLIT;
   if (split < s_first || split > s_last) return;
   const int lo = max(split * SPLIT, start[0] / 16 * 16);
   const int hi = min((split + 1) * SPLIT, pos[0] + 1);  // keys [lo, hi), not empty
-  const int* table = block_tables + (int64_t)tok_seq[tok] * max_blocks;
+  const int* table = block_tables + (int64_t)work.z * max_blocks;
   const int g = nh / nkv;
   // (the wavefront's number as a scalar, so that its pages' table entries come by scalar loads)
   const int lane = threadIdx.x % PAE_WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE);
@@ -241,15 +243,15 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 template <int HD, int TPW>
 __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
                                          const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                                         int max_splits, const int* __restrict__ dec_tok,
-                                         const int* __restrict__ positions, int nh, int nkv, int window) {
+                                         int max_splits, const int4* __restrict__ dec_work, int nh, int nkv,
+                                         int window) {
   // blockDim = (items rounded up to wavefronts, G): the splits are dealt out to G groups of threads,
   // whose loads are all in flight together; group 0 then adds the groups' sums in group order.
   extern __shared__ float s_merge[];  // [G - 1][items][6]: four sums, maximum, sum of weights
   constexpr int SPLIT = 64 * TPW;
   const int kvh = blockIdx.x;
-  const int tok = dec_tok[blockIdx.y];
-  const int pos = positions[tok];
+  const int4 work = dec_work[blockIdx.y];
+  const int tok = work.x, pos = work.y;
   const int start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int s_first = start / SPLIT, nsplits = pos / SPLIT - s_first + 1;
   const int g = nh / nkv, items = g * (HD / 4);
@@ -612,12 +614,13 @@ static int check_common(const char* what, int nh, int nkv, int hd, int bs, int m
 #define DECODE_TPW 2
 extern "C" int pae_attn_decode_split() { return 64 * DECODE_TPW; }
 
+// dec_work[i] = (flat row of the token, its position, row of its sequence in block_tables, unused),
+// 16 bytes each, 16-byte aligned.
 // Workspace: part_acc holds num_dec * nh * max_splits * hd floats, part_ml num_dec * nh * max_splits * 2,
 // max_splits = ceil(max_blocks * bs / pae_attn_decode_split()).
 extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
-                                    const void* k_cache, const void* v_cache, const int* dec_tok, int num_dec,
-                                    const int* positions, const int* tok_seq, const int* block_tables,
-                                    int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
+                                    const void* k_cache, const void* v_cache, const int* dec_work, int num_dec,
+                                    const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
                                     void* part_acc, void* part_ml, hipStream_t stream) {
   if (int rc = check_common("attn_decode", nh, nkv, hd, bs, max_blocks, window)) return rc;
   PAE_REQUIRE(num_dec <= 65535 && nkv <= 65535, "attn_decode: grid too large");
@@ -638,10 +641,10 @@ extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q
 #define CALL(HD)                                                                                            \
   attn_decode_kernel<HD, DECODE_TPW><<<grid, 256, (size_t)3 * (HD / 4 + 2) * PAE_WAVE * sizeof(float), stream>>>( \
       (float*)part_acc, (float*)part_ml, max_splits, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,     \
-      (const bf16_t*)v_cache, dec_tok, positions, tok_seq, block_tables, max_blocks, bs, nh, nkv, scale_log2, \
+      (const bf16_t*)v_cache, (const int4*)dec_work, block_tables, max_blocks, bs, nh, nkv, scale_log2, \
       window);                                                                                               \
   attn_decode_merge_kernel<HD, DECODE_TPW><<<merge_grid, dim3(merge_x, merge_groups), merge_lds, stream>>>( \
-      (bf16_t*)out, out_stride, (const float*)part_acc, (const float*)part_ml, max_splits, dec_tok, positions, \
+      (bf16_t*)out, out_stride, (const float*)part_acc, (const float*)part_ml, max_splits, (const int4*)dec_work, \
       nh, nkv, window)
   FOR_HEAD_DIM(hd, CALL)
 #undef CALL

@@ -167,7 +167,10 @@ class StepRunner:
         flat = array("i", ids)
         for piece in (positions, tok_seq, slots, rows, fed_places, fed_rows):
             flat.extend(piece)
+        list_offsets = []
         for _, _, values, _ in part_lists:
+            flat.extend([0] * (-len(flat) % 4))  # every part's list starts on a 16-byte boundary
+            list_offsets.append(len(flat))
             flat.extend(values)
         for width, tables in zip(widths, per_group):
             hole = array("i", [-1])
@@ -203,7 +206,8 @@ class StepRunner:
         d_ids, d_pos, d_seq, d_slots, d_rows = take(T), take(T), take(T), take(S), take(len(rows))
         d_fed_places, d_fed_rows = take(S), take(S)
         memo: Dict[object, object] = {}
-        for key, name, values, width in part_lists:
+        for (key, name, values, width), at in zip(part_lists, list_offsets):
+            off = at
             tensor = take(len(values))
             memo.setdefault(key, {})[name] = tensor.view(-1, width) if width else tensor
         if fed:

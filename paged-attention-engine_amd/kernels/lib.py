@@ -70,7 +70,7 @@ def _declare(lib) -> None:
         "pae_sample_chunks": [I],
         "pae_sample_static": [P, P, L, P, P, I, I, P],
         "pae_sample_static_slots": [],
-        "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, P, P],
+        "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, P, P, P],
         "pae_attn_decode_split": [],
         "pae_attn_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
     }
@@ -517,27 +517,27 @@ def mfma_attention_supported(dtype: torch.dtype, nh: int, nkv: int, hd: int, bs:
 
 
 def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
-                dec_tok: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
-                block_tables: torch.Tensor, nh: int, nkv: int, hd: int, scale: float, window: int) -> None:
-    """Attention of the single new token of each sequence listed in `dec_tok` (flat
-    token indices) over that sequence's cached keys: split over the keys, then merged."""
-    _gpu(out, q, k_cache, v_cache, dec_tok, positions, tok_seq, block_tables)
-    n = dec_tok.numel()
+                dec_work: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, hd: int, scale: float,
+                window: int) -> None:
+    """Attention of the single new token of each sequence listed in `dec_work` over that sequence's
+    cached keys: split over the keys, then merged.  dec_work[i] = (flat row of the token, its
+    position, row of its sequence in `block_tables`, 0)."""
+    _gpu(out, q, k_cache, v_cache, dec_work, block_tables)
     bs = k_cache.shape[2]
     assert q.dtype == torch.bfloat16 == out.dtype == k_cache.dtype and q.stride(1) == 1 and out.stride(1) == 1
     assert q.shape[1] >= nh * hd and out.shape[1] >= nh * hd and out.shape[0] == q.shape[0]
     _check_pools(k_cache, v_cache, nkv, bs, hd)
-    assert dec_tok.dtype == torch.int32 and positions.dtype == torch.int32 and tok_seq.dtype == torch.int32
-    assert positions.numel() == q.shape[0] == tok_seq.numel()
+    assert dec_work.dtype == torch.int32 and dec_work.dim() == 2 and dec_work.shape[1] == 4 and dec_work.is_contiguous()
+    assert dec_work.data_ptr() % 16 == 0, "the decode work list must start on a 16-byte boundary"
+    n = dec_work.shape[0]
     assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
     max_splits = -(-block_tables.shape[1] * bs // library().pae_attn_decode_split())
     part_acc = torch.empty((n * nh * max_splits, hd), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n * nh * max_splits, 2), dtype=torch.float32, device=q.device)
     _check(library().pae_attn_decode_bf16(
         out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
-        dec_tok.data_ptr(), n, positions.data_ptr(), tok_seq.data_ptr(), block_tables.data_ptr(),
-        block_tables.shape[1], bs, nh, nkv, hd, float(scale), int(window),
-        part_acc.data_ptr(), part_ml.data_ptr(), _stream()))
+        dec_work.data_ptr(), n, block_tables.data_ptr(), block_tables.shape[1], bs, nh, nkv, hd, float(scale),
+        int(window), part_acc.data_ptr(), part_ml.data_ptr(), _stream()))
 
 
 PREFILL_TILE = 64  # tokens per run of the prefill attention kernel (one workgroup each)

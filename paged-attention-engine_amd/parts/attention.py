@@ -31,11 +31,13 @@ WORK_LISTS = ("paged attention work lists", K.PREFILL_TILE)
 
 
 def attention_work_lists(shape: StepShape):
-    """What the matrix-core attention kernels walk: `decode_tokens`, the flat rows of sequences that
-    bring one token, and `prefill_tiles`, runs of up to PREFILL_TILE consecutive tokens of the
+    """What the matrix-core attention kernels walk: `decode_work`, one (flat row, position, table
+    row, 0) for every sequence that brings one token (all a workgroup needs to know of its token in
+    one 16-byte load), and `prefill_tiles`, runs of up to PREFILL_TILE consecutive tokens of the
     others as (table row, first flat token, count).  The runs with the most keys come first:
     workgroups start in list order, and the last to finish sets the kernel's time."""
-    decode_tokens = [start for start, n in zip(shape.q_starts, shape.q_lens) if n == 1]
+    decode_work = [x for row, (start, n, past) in enumerate(zip(shape.q_starts, shape.q_lens, shape.past_lens))
+                   if n == 1 for x in (start, past, row, 0)]
     runs = []
     for row, (start, n, past) in enumerate(zip(shape.q_starts, shape.q_lens, shape.past_lens)):
         if n > 1:
@@ -43,7 +45,7 @@ def attention_work_lists(shape: StepShape):
                 count = min(K.PREFILL_TILE, n - first)
                 runs.append((past + first + count, (row, start + first, count)))
     runs.sort(key=lambda run: -run[0])
-    return {"decode_tokens": (decode_tokens, 0), "prefill_tiles": ([x for _, tile in runs for x in tile], 3)}
+    return {"decode_work": (decode_work, 4), "prefill_tiles": ([x for _, tile in runs for x in tile], 3)}
 
 
 @register_mixer("attention")
@@ -151,9 +153,9 @@ class PagedAttention(Part):
         geometry = (s.num_heads, s.num_kv_heads, s.head_dim, s.scale, s.window or 0)
         work = ctx.memo.get(WORK_LISTS) if self._matrix_cores(ctx.cache.block_size) else None
         if work is not None:
-            decode_tokens, prefill_tiles = work["decode_tokens"], work["prefill_tiles"]
-            if decode_tokens.numel():
-                K.attn_decode(attn, qkv, k_cache, v_cache, decode_tokens, ctx.positions, ctx.tok_seq, table, *geometry)
+            decode_work, prefill_tiles = work["decode_work"], work["prefill_tiles"]
+            if decode_work.numel():
+                K.attn_decode(attn, qkv, k_cache, v_cache, decode_work, table, *geometry)
             if prefill_tiles.numel():
                 K.attn_prefill(attn, qkv, k_cache, v_cache, prefill_tiles, ctx.positions, table, *geometry)
         else:

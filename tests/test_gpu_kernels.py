@@ -530,14 +530,14 @@ def run_attention(kind, dtype, nh, nkv, hd, bs, window, seq_lens, q_lens, sharp=
         K().paged_attention_generic(out, qd, d(kp), d(vp), pos_d, seq_d, tab_d, nh, nkv, hd, scale, window)
     else:
         starts = [sum(q_lens[:s]) for s in range(len(q_lens))]
-        dec = [starts[s] for s in range(len(q_lens)) if q_lens[s] == 1]
+        dec = [[starts[s], positions[starts[s]], s, 0] for s in range(len(q_lens)) if q_lens[s] == 1]
         tiles = []
         for s, ql in enumerate(q_lens):
             if ql > 1:
                 for first in range(0, ql, K().PREFILL_TILE):
                     tiles.append([s, starts[s] + first, min(K().PREFILL_TILE, ql - first)])
         if dec:
-            K().attn_decode(out, qd, d(kp), d(vp), d(dec, torch.int32), pos_d, seq_d, tab_d, nh, nkv, hd, scale, window)
+            K().attn_decode(out, qd, d(kp), d(vp), d(dec, torch.int32), tab_d, nh, nkv, hd, scale, window)
         if tiles:
             K().attn_prefill(out, qd, d(kp), d(vp), d(tiles, torch.int32), pos_d, tab_d, nh, nkv, hd, scale, window)
     return out.double().cpu(), want
