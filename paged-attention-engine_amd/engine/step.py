@@ -13,6 +13,7 @@ reserved room for every token (:414-417), so positions are the run
 
 from __future__ import annotations
 
+import os
 from array import array
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -77,6 +78,9 @@ class StepRunner:
         self._graphs: Dict[tuple, _CapturedStep] = {}
         self.graph_replays = 0
         self.graph_recordings = 0
+        # a slow check for tests and debugging: after every step, wait for the device and see that the
+        # products' ticket counters are back at zero
+        self.check_tickets = bool(os.environ.get("PAE_CHECK_TICKETS"))
 
     def run(self, entries: Sequence[StepEntry],
             feeds: Optional[Tuple[torch.Tensor, Sequence[Tuple[int, int]]]] = None) -> torch.Tensor:
@@ -221,7 +225,10 @@ class StepRunner:
                           cache=cache, seq_ids=seq_ids, q_starts=q_starts, q_lens=q_lens,
                           past_lens=past_lens, host_slots=slots, memo=memo)
         if captured is None:
-            return self.model.forward(ctx, d_ids, d_rows)
+            logits = self.model.forward(ctx, d_ids, d_rows)
+            if self.check_tickets:
+                K.check_tickets_zero(self.device)
+            return logits
         if captured.graph is None:
             # record the step: nothing runs during the recording, so replay it right away
             graph = torch.cuda.CUDAGraph()
@@ -233,4 +240,6 @@ class StepRunner:
             self.model.forward_pass_count += 1
         captured.graph.replay()
         self.graph_replays += 1
+        if self.check_tickets:
+            K.check_tickets_zero(self.device)
         return captured.logits[:R]

@@ -385,25 +385,40 @@ def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optio
     bp, bf = _param(bias)
     sp, st, se = _row_scale(row_scale, M, K_)
     parts, counters = _ticket_scratch(a.device, M, N, splits if epilogue != EPI_F32 else 1)
-    _check(library().pae_gemm_skinny(epilogue, out.data_ptr(), out.stride(-2), a.data_ptr(), a.stride(0),
-                                     w.data_ptr(), bp, bf, M, N, K_, splits, M * N, _ptr(parts), _ptr(counters),
-                                     sp, st, se, nr, ld_next, nw, nwf, ns, _stream()))
+    _launch_ticketed(counters, lambda: library().pae_gemm_skinny(
+        epilogue, out.data_ptr(), out.stride(-2), a.data_ptr(), a.stride(0), w.data_ptr(), bp, bf, M, N, K_, splits,
+        M * N, _ptr(parts), _ptr(counters), sp, st, se, nr, ld_next, nw, nwf, ns, _stream()))
 
 
-_TICKETS: dict = {}
+_TICKETS: dict = {}        # device index -> counters
+_TICKET_STREAM: dict = {}  # device index -> the stream whose launches use them
 
 
 def skinny_tickets(device) -> torch.Tensor:
-    """The zeroed counters of products whose k ranges are added up inside the kernel (every launch
-    leaves them zero; launches on one device run one after the other and share them).  Made at the
-    first call for a device, which must not come while a graph records: a model asks when it is
-    bound."""
+    """The zeroed counters of products whose k ranges are added up inside the kernel.  Every launch
+    leaves them zero, and launches share them, so they must run one after the other: the counters
+    belong to the stream that is current when they are made (a model asks when it is bound, before
+    any step is recorded as a graph), and `_ticket_scratch` refuses launches from another stream.
+    Recording a graph on torch's capture stream is not a launch; its replays are, on the stream
+    they are replayed on."""
     index = torch.device(device).index or 0
     if index not in _TICKETS:
         if torch.cuda.is_current_stream_capturing():
             raise KernelError("the ticket counters must exist before a graph is recorded")
         _TICKETS[index] = torch.zeros(1 << 16, dtype=torch.int32, device=device)
+        _TICKET_STREAM[index] = torch.cuda.current_stream(device).cuda_stream
     return _TICKETS[index]
+
+
+def check_tickets_zero(device) -> None:
+    """Raise unless every ticket counter is zero (it waits for the device: a check for tests and
+    for runs with PAE_CHECK_TICKETS set, after each step)."""
+    index = torch.device(device).index or 0
+    counters = _TICKETS.get(index)
+    if counters is not None and bool(counters.any()):
+        where = counters.nonzero().flatten()[:8].tolist()
+        raise KernelError(f"ticket counters {where} are not zero between launches: a product with k ranges "
+                          "was cut short, or launches from two streams overlapped")
 
 
 def _ticket_scratch(device, M: int, N: int, splits: int):
@@ -411,9 +426,25 @@ def _ticket_scratch(device, M: int, N: int, splits: int):
     if splits <= 1:
         return None, None
     lib, counters = library(), skinny_tickets(device)
+    index = torch.device(device).index or 0
+    if (not torch.cuda.is_current_stream_capturing()
+            and torch.cuda.current_stream(device).cuda_stream != _TICKET_STREAM[index]):
+        raise KernelError("products with k ranges share their ticket counters and must all be launched on the "
+                          "stream the counters were made on; this launch comes from another stream")
     if lib.pae_skinny_ticket_slots(M, N) > counters.numel():
         raise KernelError(f"{N} weight rows by {M} rows need more ticket counters than there are")
     return torch.empty(lib.pae_skinny_ticket_floats(M, N, splits), dtype=torch.float32, device=device), counters
+
+
+def _launch_ticketed(counters, call) -> None:
+    """Run a launch that uses the ticket counters; if it is refused or fails, the counters are put
+    back to zero before the error goes up (a later product would otherwise add up the wrong ranges)."""
+    try:
+        _check(call())
+    except KernelError:
+        if counters is not None and not torch.cuda.is_current_stream_capturing():
+            counters.zero_()
+        raise
 
 
 def whole_sum_splits(N: int, K: int, M: int) -> int:
@@ -470,11 +501,10 @@ def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias
     splits = 1 if splits is None else splits
     parts, counters = _ticket_scratch(a.device, M, N, splits)
     sp, st, se = _row_scale(row_scale, M, K_)
-    _check(lib.pae_gemm_skinny_rope(q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(),
-                                    bp, bf, M, K_, nh, nkv, hd, rot, _ptr(cos_sin) if rot else None,
-                                    positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks,
-                                    block_size, _ptr(k_cache), _ptr(v_cache), splits, _ptr(parts), _ptr(counters),
-                                    sp, st, se, _stream()))
+    _launch_ticketed(counters, lambda: lib.pae_gemm_skinny_rope(
+        q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(), bp, bf, M, K_, nh, nkv, hd, rot,
+        _ptr(cos_sin) if rot else None, positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks,
+        block_size, _ptr(k_cache), _ptr(v_cache), splits, _ptr(parts), _ptr(counters), sp, st, se, _stream()))
 
 
 def gemm_plain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:

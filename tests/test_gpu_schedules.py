@@ -238,3 +238,41 @@ def test_ignoring_the_block_tables_diverges_on_a_fragmented_pool(tmp_path, dtype
     helpers.check_logits(run(False), want, dtype, "E", "through the real tables")
     off = float((run(True) - want).abs().max())
     assert off > 10 * bound, f"identity tables moved the logits by {off:.3e} only (bound {bound:.3e})"
+
+
+def test_ticket_counters_are_zero_between_steps_and_belong_to_one_stream(tmp_path):
+    """Products whose k ranges are added up inside the kernel share counters that every launch
+    leaves at zero.  With the runner's check switched on, every step of a run at widths that use k
+    ranges (prefill portions of 17 to 64 rows, decode steps, a padded recorded step) is followed by
+    a look at the counters; and a launch from a second stream is refused instead of racing."""
+    from paged_attention_engine_amd.kernels import lib as K
+
+    cfg = dict(helpers.TINY_E, hidden_size=2048, intermediate_size=4096, num_attention_heads=16,
+               num_key_value_heads=2, head_dim=128, use_sliding_window=False)
+    model = pae.random_model(cfg, 3, "bfloat16")
+    cache = model.new_cache(16, 64, 12)
+    runner = pae.StepRunner(model, cache)
+    runner.check_tickets = True
+    ids = {s: tokens_of(cfg, 80, 900 + s) for s in range(9)}
+    done = {s: 0 for s in ids}
+    for plan in ([(0, 40), (1, 20)], [(0, 1), (1, 1), (2, 64)], [(s, 3) for s in range(3, 9)],
+                 [(s, 1) for s in range(9)], [(s, 1) for s in range(9)]):
+        entries = []
+        for s, n in plan:
+            if not cache.has_sequence(s):
+                assert cache.create_sequence(s)
+            assert cache.reserve(s, n).ok
+            entries.append(pae.StepEntry(s, tuple(ids[s][done[s]:done[s] + n]), (n - 1,)))
+            done[s] += n
+        runner.run(entries)  # raises if a counter is left standing
+    assert runner.graph_replays >= 2
+    K.check_tickets_zero("cuda:0")
+    a = torch.randn(40, 2048, device="cuda:0").to(torch.bfloat16)
+    w = torch.randn(4096, 2048, device="cuda:0").to(torch.bfloat16)
+    out = torch.empty(40, 4096, device="cuda:0", dtype=torch.bfloat16)
+    K.gemm_skinny(out, a, w, None, K.EPI_BF16, 2)  # on the counters' own stream: fine
+    with torch.cuda.stream(torch.cuda.Stream()):
+        with pytest.raises(K.KernelError, match="another stream"):
+            K.gemm_skinny(out, a, w, None, K.EPI_BF16, 2)
+    torch.cuda.synchronize()
+    K.check_tickets_zero("cuda:0")
