@@ -21,11 +21,12 @@ int pae_add_rmsnorm(int dtype, void* residual, const void* delta, int parts, int
                     const void* weight, int w_is_f32, float eps, const int* rows, void* out, int num_rows,
                     int hidden, int write_residual, hipStream_t stream);
 int pae_residual_add(int dtype, void* residual, const void* delta, int64_t n, hipStream_t stream);
+int pae_copy_i32(int* dst, const int* src, int n, hipStream_t stream);  // src: device or pinned host memory
 int pae_scatter_i32(int* dst, const int* dst_idx, const int* src, const int* src_idx, int n, hipStream_t stream);
 int pae_rope_table(float* cos_sin, const int* positions, const float* inv_freq, int num_tokens, int half,
                    hipStream_t stream);
 int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int rot,
-                      const float* cos_sin, const int* positions, const int* tok_seq, const int* block_tables,
+                      const void* bias, int b_is_f32, const float* cos_sin, const int* positions, const int* tok_seq, const int* block_tables,
                       int max_blocks, int bs, void* k_cache, void* v_cache, int write_kv, hipStream_t stream);
 int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, int block, hipStream_t stream);
 int pae_gemm_plain(int in_dtype, int out_dtype, void* C, int64_t ldc, const void* A, int64_t lda, const void* W,

@@ -343,6 +343,22 @@ extern "C" int pae_scatter_i32(int* dst, const int* dst_idx, const int* src, con
   return pae_check_launch("scatter_i32");
 }
 
+// dst[i] = src[i].  `src` may be pinned host memory, which the GPU reads over the bus: a step's few
+// kilobytes of metadata reach the device by this kernel, in line with the kernels that need them,
+// instead of through the copy engine, whose hand-over from and to the compute queue leaves the
+// GPU idle for a few hundred microseconds between steps.
+__global__ void copy_i32_kernel(int* __restrict__ dst, const int* __restrict__ src, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+extern "C" int pae_copy_i32(int* dst, const int* src, int n, hipStream_t stream) {
+  PAE_REQUIRE(n >= 0 && dst && src, "copy_i32: n=%d", n);
+  if (n == 0) return 0;
+  copy_i32_kernel<<<(n + 255) / 256, 256, 0, stream>>>(dst, src, n);
+  return pae_check_launch("copy_i32");
+}
+
 // ---------------------------------------------------------------- rotation + cache write
 // qkv row t holds [q heads | k heads | v heads], each head `hd` wide.  Query and
 // key heads are rotated over their first `rot` features in pairs (i, i + rot/2):
@@ -356,7 +372,8 @@ extern "C" int pae_scatter_i32(int* dst, const int* dst_idx, const int* src, con
 // values transposed within the page, [block][kv head][hd][bs].
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, int nh, int nkv, int hd,
-                                     int rot, const float* __restrict__ cos_sin,
+                                     int rot, const void* __restrict__ bias, int b_is_f32,
+                                     const float* __restrict__ cos_sin,
                                      const int* __restrict__ positions, const int* __restrict__ tok_seq,
                                      const int* __restrict__ block_tables, int max_blocks, int bs,
                                      T* __restrict__ k_cache, T* __restrict__ v_cache, int write_kv) {
@@ -373,10 +390,14 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, in
   if (write_kv) page_base = (int64_t)block_tables[(int64_t)tok_seq[t] * max_blocks + pos / bs] * nkv * head_step;
   const int half = rot / 2;
   const int rotated_heads = nh + (write_kv ? nkv : 0);
+  // with a bias, row[j] stands for round(row[j] + bias[j]): the projection's bias is added here, on
+  // the way, where the product before left it out (the sum is rounded to T before the rotation, as
+  // the projection's own bias epilogue would have rounded it)
+  auto at = [&](int j) { return bias ? round_to<T>(to_f32(row[j]) + load_param(bias, b_is_f32, j)) : to_f32(row[j]); };
   for (int idx = threadIdx.x; idx < rotated_heads * half; idx += blockDim.x) {
     const int h = idx / half, i = idx % half;
     const float c = cos_sin[((int64_t)t * half + i) * 2], s = cos_sin[((int64_t)t * half + i) * 2 + 1];
-    const float a = to_f32(row[h * hd + i]), b = to_f32(row[h * hd + i + half]);
+    const float a = at(h * hd + i), b = at(h * hd + i + half);
     const T lo = from_f32<T>(a * c - b * s), hi = from_f32<T>(b * c + a * s);
     if (h < nh) {  // queries are rotated in place
       row[h * hd + i] = lo;
@@ -387,16 +408,21 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, in
       dst[i + half] = hi;
     }
   }
+  const int tail = hd - rot;  // features beyond the rotated ones pass through
+  if (bias)  // ... but for the bias, which the queries' unrotated features still have to get
+    for (int idx = threadIdx.x; idx < nh * tail; idx += blockDim.x) {
+      const int j = (idx / tail) * hd + rot + idx % tail;
+      row[j] = from_f32<T>(at(j));
+    }
   if (!write_kv) return;
-  const int tail = hd - rot;  // features of a key beyond the rotated ones pass through
   for (int idx = threadIdx.x; idx < nkv * tail; idx += blockDim.x) {
     const int h = idx / tail, i = rot + idx % tail;
-    k_cache[page_base + h * head_step + (int64_t)off * hd + i] = k[h * hd + i];
+    k_cache[page_base + h * head_step + (int64_t)off * hd + i] = from_f32<T>(at((nh + h) * hd + i));
   }
   // values are stored transposed within a page: [block][kv head][feature][offset]
   for (int idx = threadIdx.x; idx < nkv * hd; idx += blockDim.x) {
     const int h = idx / hd, i = idx % hd;
-    v_cache[page_base + h * head_step + (int64_t)i * bs + off] = v[h * hd + i];
+    v_cache[page_base + h * head_step + (int64_t)i * bs + off] = from_f32<T>(at((nh + nkv + h) * hd + i));
   }
 }
 
@@ -422,7 +448,8 @@ extern "C" int pae_rope_table(float* cos_sin, const int* positions, const float*
 }
 
 extern "C" int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv,
-                                 int hd, int rot, const float* cos_sin, const int* positions,
+                                 int hd, int rot, const void* bias, int b_is_f32, const float* cos_sin,
+                                 const int* positions,
                                  const int* tok_seq, const int* block_tables, int max_blocks, int bs,
                                  void* k_cache, void* v_cache, int write_kv, hipStream_t stream) {
   PAE_REQUIRE(nh > 0 && nkv >= 0 && hd > 0, "rope_kv_write: bad head sizes nh=%d nkv=%d hd=%d", nh, nkv, hd);
@@ -434,12 +461,12 @@ extern "C" int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int n
   if (num_tokens <= 0) return 0;
   if (dtype == PAE_F32)
     rope_kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>(
-        (float*)qkv, row_stride, nh, nkv, hd, rot, cos_sin, positions, tok_seq, block_tables, max_blocks, bs,
-        (float*)k_cache, (float*)v_cache, write_kv);
+        (float*)qkv, row_stride, nh, nkv, hd, rot, bias, b_is_f32, cos_sin, positions, tok_seq, block_tables,
+        max_blocks, bs, (float*)k_cache, (float*)v_cache, write_kv);
   else if (dtype == PAE_BF16)
     rope_kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
-        (bf16_t*)qkv, row_stride, nh, nkv, hd, rot, cos_sin, positions, tok_seq, block_tables, max_blocks, bs,
-        (bf16_t*)k_cache, (bf16_t*)v_cache, write_kv);
+        (bf16_t*)qkv, row_stride, nh, nkv, hd, rot, bias, b_is_f32, cos_sin, positions, tok_seq, block_tables,
+        max_blocks, bs, (bf16_t*)k_cache, (bf16_t*)v_cache, write_kv);
   else
     return pae_fail("rope_kv_write: unknown dtype code %d", dtype);
   return pae_check_launch("rope_kv_write");

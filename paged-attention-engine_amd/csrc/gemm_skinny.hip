@@ -283,10 +283,23 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
 // whichever workgroup it is (so the sums do not depend on the order of arrival), puts the counter
 // back to zero and runs the epilogue.  Nobody waits for anybody.
 //
-// Workgroups run on several dies, each with an L2 of its own, so the partials are written and read
-// as device-scope atomic accesses, which go past the caches to memory, and a workgroup draws its
-// ticket only when its stores have been acknowledged.  (Ordinary stores followed by a device-scope
-// fence do the same, but the fence writes back the die's whole L2: measured at 13 us a launch.)
+// Why relaxed device-scope atomics and one wait are enough here (gfx942/gfx950).  The chip is eight
+// dies, each with an L2 of its own that is not kept coherent with the others'; the memory side behind
+// them (the shared last-level cache and HBM) is the point at which all dies agree.  A device-scope
+// ("agent") atomic store or load is issued with the sc1 bit: the store is written through to that
+// point and the load is served from it, whatever either die's L2 holds.  `s_waitcnt vmcnt(0)` returns
+// when every vector memory operation of the wavefront, these stores included, has been
+// acknowledged, which for a written-through store means that it has arrived there.  So: (1) a
+// workgroup's partial sums are at the common point before it draws its ticket; (2) the ticket is a
+// device-scope read-modify-write, carried out at the same point, so tickets are handed out in one
+// order, and whoever draws the last one does so after every other range's partials have arrived;
+// (3) its loads of the partials are issued after the ticket's value has come back (they sit behind a
+// branch on that value and a compiler barrier) and, being sc1 loads, cannot be served stale from a
+// cache.  A release fence would add a write-back of the die's whole L2 (`buffer_wbl2`) for the sake
+// of ordinary stores that may still be dirty there; there are none that matter, because the
+// partials never were ordinary stores (measured: 13 us a launch with the fence, 1 us without).
+// The counters are shared by every launch on a device: the launches must not overlap, which the
+// host side enforces by tying the counters to one stream.
 struct SkinnyTickets {
   float* parts;   // [slots][k ranges][RT * 4][64]: a wavefront's accumulators, lane by lane
   int* counters;  // [slots], zero before and after every launch; null: one k range

@@ -81,6 +81,33 @@ class StepRunner:
         # a slow check for tests and debugging: after every step, wait for the device and see that the
         # products' ticket counters are back at zero
         self.check_tickets = bool(os.environ.get("PAE_CHECK_TICKETS"))
+        # pinned staging buffers that take turns, each with the event behind which the GPU has read it
+        self._staging: List[Optional[torch.Tensor]] = [None] * self.STAGING_BUFFERS
+        self._staging_read: List[Optional[torch.cuda.Event]] = [None] * self.STAGING_BUFFERS
+        self._staging_turn = 0
+
+    STAGING_BUFFERS = 4
+
+    def _to_device(self, flat: array, dst: Optional[torch.Tensor]) -> torch.Tensor:
+        """A step's metadata to the device: into one of a few pinned buffers that take turns, and from
+        there by a small kernel in line with the step's own kernels (no trip through the copy engine,
+        no pinned allocation per step).  `dst`: the recorded step's input buffer, or None for a new one."""
+        n = len(flat)
+        turn = self._staging_turn
+        self._staging_turn = (turn + 1) % self.STAGING_BUFFERS
+        if self._staging_read[turn] is not None:
+            self._staging_read[turn].synchronize()  # the step that used this buffer has read it (long ago)
+        pinned = self._staging[turn]
+        if pinned is None or pinned.numel() < n:
+            pinned = self._staging[turn] = torch.empty(max(1024, 2 * n), dtype=torch.int32, pin_memory=True)
+        pinned[:n].copy_(torch.frombuffer(flat, dtype=torch.int32))
+        if dst is None:
+            dst = torch.empty(n, dtype=torch.int32, device=self.device)
+        K.copy_int32_from_pinned(dst, pinned, n)
+        if self._staging_read[turn] is None:
+            self._staging_read[turn] = torch.cuda.Event()
+        self._staging_read[turn].record()
+        return dst
 
     def run(self, entries: Sequence[StepEntry],
             feeds: Optional[Tuple[torch.Tensor, Sequence[Tuple[int, int]]]] = None) -> torch.Tensor:
@@ -161,7 +188,7 @@ class StepRunner:
         part_lists = [(key, name, list(flat), width) for key, part in self._list_parts.items()
                       for name, (flat, width) in part.step_lists(shape).items()]
 
-        # one staging buffer, one copy to the device
+        # one staging buffer, one copy to the device (see `_to_device`)
         # places and rows of token ids that come from the device, padded to one per sequence
         fed = list(feeds[1]) if feeds is not None else []
         if len(fed) > S or any(not (0 <= place < T and 0 <= row < feeds[0].numel()) for place, row in fed):
@@ -181,7 +208,6 @@ class StepRunner:
             for table in tables:
                 flat.extend(table)
                 flat.extend(hole * (width - len(table)))
-        staging = torch.frombuffer(flat, dtype=torch.int32).pin_memory()
 
         captured = None
         if decode_only:
@@ -195,10 +221,9 @@ class StepRunner:
                     self._graphs.pop(next(iter(self._graphs)))
                 captured = _CapturedStep(torch.empty(len(flat), dtype=torch.int32, device=self.device))
             self._graphs[key] = captured  # last used, last to go
-            captured.inputs.copy_(staging, non_blocking=True)
-            dev = captured.inputs
+            dev = self._to_device(flat, captured.inputs)
         else:
-            dev = staging.to(self.device, non_blocking=True)
+            dev = self._to_device(flat, None)
         off = 0
 
         def take(count):

@@ -56,8 +56,9 @@ def _declare(lib) -> None:
         "pae_add_rmsnorm": [I, P, P, I, L, P, I, F, P, P, I, I, I, P],
         "pae_residual_add": [I, P, P, L, P],
         "pae_scatter_i32": [P, P, P, P, I, P],
+        "pae_copy_i32": [P, P, I, P],
         "pae_rope_table": [P, P, P, I, I, P],
-        "pae_rope_kv_write": [I, P, L, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P],
+        "pae_rope_kv_write": [I, P, L, I, I, I, I, I, P, I, P, P, P, P, I, I, P, P, I, P],
         "pae_swiglu": [I, P, P, I, I, I, P],
         "pae_gemm_skinny": [I, P, L, P, L, P, P, I, I, I, I, I, L, P, P, P, I, F, P, L, P, I, P, P],
         "pae_gemm_skinny_rope": [P, L, P, L, P, P, I, I, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P, P, P, I, F, P],
@@ -187,6 +188,15 @@ def residual_add(residual: torch.Tensor, delta: torch.Tensor) -> None:
                                       residual.numel(), _stream()))
 
 
+def copy_int32_from_pinned(dst: torch.Tensor, src: torch.Tensor, n: int) -> None:
+    """dst[:n] = src[:n] by a kernel on the current stream; `src` is pinned host memory (which the
+    GPU reads in place) and must stay as it is until the kernel has run."""
+    _gpu(dst)
+    assert dst.dtype == torch.int32 == src.dtype and dst.is_contiguous() and src.is_contiguous()
+    assert src.is_pinned() and 0 <= n <= min(dst.numel(), src.numel())
+    _check(library().pae_copy_i32(dst.data_ptr(), src.data_ptr(), n, _stream()))
+
+
 def scatter_int32(dst: torch.Tensor, dst_idx: torch.Tensor, src: torch.Tensor, src_idx: torch.Tensor, n: int) -> None:
     """dst[dst_idx[i]] = src[src_idx[i]] for i < n (int32 everywhere; the index lists may be longer than n).
     The caller vouches for the indices: they are not checked on the device."""
@@ -216,12 +226,16 @@ def _check_cos_sin(cos_sin: Optional[torch.Tensor], rot: int, T: int) -> None:
 
 def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, cos_sin: Optional[torch.Tensor],
                   positions: torch.Tensor, tok_seq: Optional[torch.Tensor], block_tables: Optional[torch.Tensor],
-                  block_size: int, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor]) -> None:
+                  block_size: int, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                  bias: Optional[torch.Tensor] = None) -> None:
     """Rotate the query heads of `qkv` in place by the angles whose cosines and sines `cos_sin`
     holds ([T, rot / 2, 2], see `rope_table`); rotate the key heads and copy the value heads
     into their cache slots (skipped when `k_cache` is None: then the row holds query heads only
-    and nkv must be 0)."""
-    _gpu(qkv, cos_sin, positions, tok_seq, block_tables, k_cache, v_cache)
+    and nkv must be 0).  With `bias` (one value per feature of the row) the row stands for the
+    projection without its bias, which is added here first."""
+    _gpu(qkv, cos_sin, positions, tok_seq, block_tables, k_cache, v_cache, bias)
+    if bias is not None:
+        assert bias.numel() == (nh + 2 * nkv) * hd
     T = qkv.shape[0]
     assert qkv.dim() == 2 and qkv.stride(1) == 1 and positions.dtype == torch.int32 and positions.numel() == T
     write = k_cache is not None
@@ -233,8 +247,9 @@ def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, cos_s
         assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
         _check_pools(k_cache, v_cache, nkv, block_size, hd)
         max_blocks = block_tables.shape[1]
+    bp, bf = _param(bias)
     _check(library().pae_rope_kv_write(code_of(qkv.dtype), qkv.data_ptr(), qkv.stride(0), T, nh, nkv, hd, rot,
-                                       _ptr(cos_sin) if rot else None, positions.data_ptr(), _ptr(tok_seq),
+                                       bp, bf, _ptr(cos_sin) if rot else None, positions.data_ptr(), _ptr(tok_seq),
                                        _ptr(block_tables), max_blocks, block_size, _ptr(k_cache), _ptr(v_cache),
                                        1 if write else 0, _stream()))
 

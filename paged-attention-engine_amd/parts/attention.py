@@ -138,9 +138,14 @@ class PagedAttention(Part):
                                ctx.positions, ctx.tok_seq, table, bs, k_cache, v_cache, splits,
                                row_scale=owed.row_scale if owed is not None else None)
             return q
-        qkv = linear(owed if owed is not None else x)
+        # many rows: the library's plain product (its variant with a bias costs the host six times the
+        # call), and the bias is added by the kernel that rotates and stores, which follows anyway
+        qkv = linear.without_bias(x) if owed is None else None
+        bias = linear.bias if qkv is not None else None
+        if qkv is None:
+            qkv = linear(owed if owed is not None else x)
         K.rope_kv_write(qkv, s.num_heads, nkv, s.head_dim, rot, cos_sin, ctx.positions, ctx.tok_seq, table, bs,
-                        k_cache, v_cache)
+                        k_cache, v_cache, bias)
         return qkv
 
     def forward(self, ctx, x):

@@ -42,9 +42,9 @@ class Linear:
     def graph_max_rows(self):
         return rows_a_graph_may_hold(self.weight.dtype, self.in_features)
 
-    def _library(self, x: torch.Tensor) -> torch.Tensor:
+    def _library(self, x: torch.Tensor, with_bias: bool = True) -> torch.Tensor:
         out = torch.empty((x.shape[0], self.out_features), dtype=x.dtype, device=x.device)
-        bias = self.bias
+        bias = self.bias if with_bias else None
         if bias is None:
             torch.mm(x, self.weight.t(), out=out)
         else:
@@ -70,6 +70,15 @@ class Linear:
             K.gemm_skinny(out, x, self.weight, self.bias, K.EPI_BF16)
             return out
         return self._library(x)
+
+    def without_bias(self, x) -> Optional[torch.Tensor]:
+        """The product without its bias where that is the cheaper call (the matrix library's plain
+        product, many rows), for a caller that adds the bias in a kernel of its own that follows
+        anyway; None where the bias costs nothing (this engine's own products)."""
+        if (self.bias is None or isinstance(x, OwedRows) or x.dtype != torch.bfloat16 or x.shape[0] == 0
+                or K.skinny_supported(x, self.weight)):
+            return None
+        return self._library(x, with_bias=False)
 
     def branch(self, x: torch.Tensor, sink=None) -> Optional[torch.Tensor]:
         """The product as a residual branch's output: [M, N] in x's dtype, or float32

@@ -378,7 +378,10 @@ def test_rope_table():
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nh,nkv,hd,rot,bs", [(4, 2, 16, 16, 4), (6, 1, 48, 48, 16), (3, 3, 32, 16, 8)])
-def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs):
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs, with_bias):
+    """`with_bias`: the rows come without the projection's bias, which the kernel adds first (rounded
+    to the storage type, as the projection's own epilogue would) before it rotates and stores."""
     torch.manual_seed(2)
     theta = 50000.0
     # two sequences: one brings positions 5..11, the other the single position 37
@@ -392,8 +395,12 @@ def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs):
     kp = torch.full((40, nkv, bs, hd), 7.0, dtype=DT[dtype])
     vp = torch.full((40, nkv, hd, bs), 7.0, dtype=DT[dtype])
     d_qkv, d_kp, d_vp = qkv.to(DEV), kp.to(DEV), vp.to(DEV)
+    bias = torch.randn((nh + 2 * nkv) * hd).to(DT[dtype]) if with_bias else None
     K().rope_kv_write(d_qkv, nh, nkv, hd, rot, table, pos_d,
-                      torch.tensor(tok_seq, dtype=torch.int32, device=DEV), tables.to(DEV), bs, d_kp, d_vp)
+                      torch.tensor(tok_seq, dtype=torch.int32, device=DEV), tables.to(DEV), bs, d_kp, d_vp,
+                      bias.to(DEV) if with_bias else None)
+    if with_bias:
+        qkv = (qkv.float() + bias.float()).to(DT[dtype])
     x = qkv.double().view(T, nh + 2 * nkv, hd)
     cos, sin = plain.rope_cos_sin(plain.rope_inv_freq(rot, theta, torch.float64), torch.tensor(positions), torch.float64)
     rotated = x.clone()
