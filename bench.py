@@ -38,6 +38,15 @@ QWEN25_1P5B = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=28, hid
                    vocab_size=151936, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
                    use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu")
 FULL_LAYERS = 28
+# Other shapes of the same architecture (--model): the 7B and 72B layer sizes, for decode steps and
+# prefills at sizes where a kernel runs longer than a launch costs.
+OTHER_SHAPES = {
+    "7b": dict(QWEN25_1P5B, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+               intermediate_size=18944, vocab_size=152064, tie_word_embeddings=False),
+    "72b": dict(QWEN25_1P5B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+                num_key_value_heads=8, intermediate_size=29568, vocab_size=152064, rms_norm_eps=1e-5,
+                tie_word_embeddings=False),
+}
 HBM_PEAK_GBS = 8000.0
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
@@ -206,7 +215,9 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--ctx", type=int, default=4096)
-    parser.add_argument("--layers", type=int, default=FULL_LAYERS)
+    parser.add_argument("--model", choices=("1.5b", "7b", "72b"), default="1.5b",
+                        help="layer sizes (default: the Qwen2.5-1.5B shape of the headline figure)")
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
     parser.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
@@ -219,14 +230,18 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
-    cfg = dict(QWEN25_1P5B, num_hidden_layers=args.layers)
+    shape = QWEN25_1P5B if args.model == "1.5b" else OTHER_SHAPES[args.model]
+    args.full_layers = shape["num_hidden_layers"]
+    args.layers = args.layers or args.full_layers
+    args.shape_name = f"Qwen2.5-{args.model.upper()} shape"
+    cfg = dict(shape, num_hidden_layers=args.layers)
     elem = 2 if args.dtype == "bfloat16" else 4
     model = build_model(cfg, args.dtype)
 
     try:
         return report(args, cfg, elem, model)
     except Unresolved as err:
-        print(json.dumps({"metric": f"decode tok/s at batch {args.batch}, context {args.ctx} (Qwen2.5-1.5B shape)",
+        print(json.dumps({"metric": f"decode tok/s at batch {args.batch}, context {args.ctx} ({args.shape_name})",
                           "value": None, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
                           "invalid": str(err)}))
         return 3
@@ -235,7 +250,7 @@ def main() -> int:
 def report(args, cfg, elem, model) -> int:
     if args.prefill_only:
         pre_s, pre_range = prefill_run(model, cfg, 2048)
-        print(json.dumps({"metric": "prefill tok/s at 2,048 tokens (Qwen2.5-1.5B shape)", "value": round(2048 / pre_s, 1),
+        print(json.dumps({"metric": f"prefill tok/s at 2,048 tokens ({args.shape_name})", "value": round(2048 / pre_s, 1),
                           "unit": "tokens/s", "ms": round(pre_s * 1e3, 3), "range_ms": round(pre_range * 1e3, 3),
                           "dtype": args.dtype,
                           "frac": round(prefill_flops(cfg, 2048) / pre_s / PEAK_FLOPS[args.dtype], 4)}))
@@ -246,17 +261,17 @@ def report(args, cfg, elem, model) -> int:
     step_bytes = weight_bytes(cfg, elem) + kv_bytes(cfg, tokens_held, elem)
     achieved = step_bytes / step_s / 1e9
     record = {
-        "metric": f"decode tok/s at batch {args.batch}, context {args.ctx} (Qwen2.5-1.5B shape)",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.ctx} ({args.shape_name})",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded uniform token ids, random weights N(0, 0.02)",
-        "config": {"model": "Qwen2.5-1.5B shape", "global_batch": args.batch, "seq_len": args.ctx,
-                   "parallelism": "single GPU", "layers": args.layers, "layers_of_model": FULL_LAYERS,
+        "config": {"model": args.shape_name, "global_batch": args.batch, "seq_len": args.ctx,
+                   "parallelism": "single GPU", "layers": args.layers, "layers_of_model": args.full_layers,
                    "hidden": cfg["hidden_size"], "q_heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
-                   "tied_head": True, "block_size": 16, "prefill_tokens": 2048},
+                   "tied_head": bool(cfg["tie_word_embeddings"]), "block_size": 16, "prefill_tokens": 2048},
         "passes": MEASURED_PASSES, "range_ms_per_step": round(step_range * 1e3, 4),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
