@@ -739,7 +739,9 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   }
   if (epilogue == EPI_RESIDUAL && mt == 1 && splits == 1 && K >= 1024) {
     // One k range, so that the sums are whole without tickets, and sixteen wavefronts to share it out:
-    // few workgroups, but each keeps its compute unit's memory pipeline full.
+    // few workgroups, but each keeps its compute unit's memory pipeline full.  (The callers choose one
+    // range where that is ahead, see kernels/lib.py `residual_splits`; for the rotating epilogue sixteen
+    // wavefronts were slower at every size tried.)
     gemm_skinny_kernel<1, 1, EPI_RESIDUAL, 4, 16><<<dim3((N + 15) / 16, 1), 1024, 0, stream>>>(
         out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, bias, b_is_f32, M, N, K, k_per_split, part_stride, rope,
         tickets, norm);

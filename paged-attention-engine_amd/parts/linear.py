@@ -94,7 +94,9 @@ class Linear:
                 weight, eps = fold
                 rows = torch.empty((x.shape[0], self.out_features), dtype=torch.bfloat16, device=x.device)
                 stats = torch.empty((x.shape[0], K.stat_tiles(self.out_features)), dtype=torch.float32, device=x.device)
-                K.gemm_skinny(residual, x, self.weight, None, K.EPI_RESIDUAL, splits, following=(rows, weight, stats))
+                K.gemm_skinny(residual, x, self.weight, None, K.EPI_RESIDUAL,
+                              K.residual_splits(self.out_features, self.in_features, x.shape[0]),
+                              following=(rows, weight, stats))
                 sink.deliver(OwedRows(rows, stats, eps))
                 return None
             out = torch.empty((splits, x.shape[0], self.out_features), dtype=torch.float32, device=x.device)
