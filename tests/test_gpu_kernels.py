@@ -377,7 +377,8 @@ def test_rope_table():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("nh,nkv,hd,rot,bs", [(4, 2, 16, 16, 4), (6, 1, 48, 48, 16), (3, 3, 32, 16, 8)])
+@pytest.mark.parametrize("nh,nkv,hd,rot,bs", [(4, 2, 16, 16, 4), (6, 1, 48, 48, 16), (3, 3, 32, 16, 8),
+                                              (12, 2, 128, 128, 16), (5, 1, 24, 8, 4), (2, 1, 20, 12, 4)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs, with_bias):
     """`with_bias`: the rows come without the projection's bias, which the kernel adds first (rounded
