@@ -343,6 +343,10 @@ def skinny_splits(N: int, K: int, M: int = 1) -> int:
         # 320 workgroups over 13,824 of k take 48 us with the norm, three ranges 35 us)
         wanted = min(8, -(-960 // tiles))
     if M > 16:
+        # every range costs its partial sums a trip to memory and back in the norm that adds them, so a
+        # workgroup wants about 128 KB of weights before another range pays (with the norm, at 64 rows:
+        # 1.5B O one range 9.8 us, six 11.5; 1.5B down four 21.0, eight 22.9; 7B O two 18.2, four 19.8)
+        wanted = max(1, min(8, round(rows * K * 2 / 131072)))
         # enough ranges of at least 1024 for the many-weight-rows kernel (128 rows a workgroup) to fill
         # the chip twice, where that many exist (72B down at 64 rows: 2 ranges 177 us, 8 ranges 115 us)
         groups = -(-N // 128)

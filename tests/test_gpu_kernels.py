@@ -103,12 +103,10 @@ def test_gemm_skinny(M, N, K_):
     out32 = torch.empty(M, N, dtype=torch.float32, device=DEV)
     K().gemm_skinny(out32, a.to(DEV), w.to(DEV), None, K().EPI_F32)
     assert (out32.double().cpu() - want).abs().max() <= 2e-5 * scale
-    splits = K().skinny_splits(N, K_, M)
-    parts = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device=DEV)
-    K().gemm_skinny(parts, a.to(DEV), w.to(DEV), None, K().EPI_F32, splits)
-    assert (parts.sum(0).double().cpu() - want).abs().max() <= 2e-5 * scale
-    if K_ >= 1536:
-        assert splits > 1
+    for splits in {K().skinny_splits(N, K_, M), 3 if K_ >= 1536 else 1}:  # the rule's choice, and three ranges
+        parts = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device=DEV)
+        K().gemm_skinny(parts, a.to(DEV), w.to(DEV), None, K().EPI_F32, splits)
+        assert (parts.sum(0).double().cpu() - want).abs().max() <= 2e-5 * scale
     # a row's result does not depend on the other rows
     if M > 1:
         one = torch.empty(1, N, dtype=torch.float32, device=DEV)
