@@ -674,9 +674,10 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   if (M == 0) return 0;
   // weight rows per workgroup: 16 for up to 8 rows of A, else 32, so that the activations, which every
   // workgroup re-reads, stay behind the weights (9 to 16 rows with 32: 7B gate/up at 16 rows 71.5 -> 61.9 us,
-  // 72B down 128.5 -> 108.6 us; at 8 rows and below 16 are as fast or faster at most sizes)
+  // 72B down 128.5 -> 108.6 us; at 8 rows and below 16 are as fast or faster at most sizes), unless that
+  // leaves too few workgroups (the QKV product of the 1.5B sizes at 16 rows: 64 workgroups, 9.2 us)
   const int mt = (M + 15) / 16;
-  const int rt = M > 8 ? 2 : 1;
+  const int rt = mt >= 2 || (M > 8 && (int64_t)((N + 31) / 32) * splits >= 128) ? 2 : 1;
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + 127) / 128 * 128;
   PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "gemm_skinny: %d k ranges are too many for K=%d", splits, K);

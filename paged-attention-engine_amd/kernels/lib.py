@@ -488,7 +488,11 @@ def whole_sum_splits(N: int, K: int, M: int) -> int:
       14B 37 -> 31 us in four, 72B 87 -> 54 us in six);
     * not with very few weight rows, where the rows of activations are shared out instead."""
     tiles, groups = -(-N // 32), -(-N // 128)
-    if M <= 16 or tiles <= 96 or 128 <= groups < 256 or groups >= 384:
+    if M <= 16:
+        # long rows of weights and not so many of them that the chip is full many times over (the QKV
+        # product of the 72B sizes): ranges of about 2,048 (at 16 rows 57 -> 45 us in four, at one row 39 -> 37 us)
+        return max(1, min(4, K // 2048)) if N <= 16384 else 1
+    if tiles <= 96 or 128 <= groups < 256 or groups >= 384:
         return 1
     if groups >= 256:
         wanted = -(-(768 if M > 48 else 512) // groups)
