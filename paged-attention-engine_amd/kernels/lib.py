@@ -334,15 +334,15 @@ def skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 def skinny_splits(N: int, K: int, M: int = 1) -> int:
     """k ranges for a product whose consumer adds float32 partials: enough workgroups to fill the
-    chip (a workgroup takes 16 weight rows, or 32 with more than 16 rows of activations)."""
-    rows = 32 if M > 16 else 16
+    chip (a workgroup takes 16 weight rows, or 32 and more with more than 8 rows of activations)."""
+    rows = 32 if M > 8 else 16
     tiles = -(-N // rows)
     wanted = max(1, min(512 // tiles, K // 256, 8))
-    if M <= 16 and tiles >= 200 and tiles * wanted < 640 and K >= 4096:
+    if M <= 8 and tiles >= 200 and tiles * wanted < 640 and K >= 4096:
         # one or two workgroups per compute unit, each with a long way to go (14B down at 8 rows:
         # 320 workgroups over 13,824 of k take 48 us with the norm, three ranges 35 us)
         wanted = min(8, -(-960 // tiles))
-    if M > 16:
+    if M > 8:
         # every range costs its partial sums a trip to memory and back in the norm that adds them, so a
         # workgroup wants about 128 KB of weights before another range pays (with the norm, at 64 rows:
         # 1.5B O one range 9.8 us, six 11.5; 1.5B down four 21.0, eight 22.9; 7B O two 18.2, four 19.8)
@@ -369,7 +369,12 @@ def residual_splits(N: int, K: int, M: int) -> int:
     range runs as sixteen wavefronts a workgroup that share out k, with no tickets and no trip to memory
     for partial sums, and is ahead wherever the 16-row workgroups fill the chip or have little to read
     (1.5B O at 8 rows 7.2 -> 5.9 us, 7B down 38.3 -> 36.1 us, 72B down 111 -> 107.5 us); a few workgroups
-    with much to read each want ranges (1.5B down: 96 workgroups of 287 KB, 17.4 us in one range, 12.5 in five)."""
+    with much to read each want ranges (1.5B down: 96 workgroups of 287 KB, 17.4 us in one range, 12.5 in five).
+    From 9 rows on the kernels for many rows are there as well, and their ranges are ahead where they are
+    more than two (at 16 rows: 7B down 42.7 us in one range, 33.2 in eight; 72B down 130 and 92)."""
+    if M > 8:
+        many = skinny_splits(N, K, M)
+        return many if many > 2 else 1
     tiles = -(-N // 16)
     if tiles >= 192 or 32 * K <= 65536:
         return 1
@@ -480,7 +485,7 @@ def _launch_ticketed(counters, call) -> None:
 
 def whole_sum_splits(N: int, K: int, M: int) -> int:
     """k ranges for a product whose epilogue needs whole sums (gate, rotation, bias), which the
-    kernel then adds up itself.  That costs a trip to memory, and pays with more than 16 rows of
+    kernel then adds up itself.  That costs a trip to memory, and pays with more than 8 rows of
     activations where workgroups are few (measured at the 1.5B to 72B layer sizes):
     * the many-weight-rows kernel with little more than one workgroup per compute unit (7B gate/up
       at 64 rows: 85 -> 72 us; with more weight rows, or somewhat fewer, one range is as fast or faster);
@@ -488,11 +493,15 @@ def whole_sum_splits(N: int, K: int, M: int) -> int:
       14B 37 -> 31 us in four, 72B 87 -> 54 us in six);
     * not with very few weight rows, where the rows of activations are shared out instead."""
     tiles, groups = -(-N // 32), -(-N // 128)
-    if M <= 16:
+    if M <= 8:
         # long rows of weights and not so many of them that the chip is full many times over (the QKV
-        # product of the 72B sizes): ranges of about 2,048 (at 16 rows 57 -> 45 us in four, at one row 39 -> 37 us)
+        # product of the 72B sizes): ranges of about 2,048 (at 8 rows 42.6 -> 40.4 us in four, at one row 39 -> 37 us)
         return max(1, min(4, K // 2048)) if N <= 16384 else 1
-    if tiles <= 96 or 128 <= groups < 256 or groups >= 384:
+    if 128 <= groups < 256:
+        # a couple of workgroups of 32 weight rows per compute unit: three ranges from 32
+        # rows on (1.5B gate/up at 64 rows 27.2 -> 23.3 us, at 32 rows 20.2 -> 19.0 us; below, one range is ahead)
+        return 3 if M >= 32 and K >= 1536 else 1
+    if tiles <= 96 or groups >= 384:
         return 1
     if groups >= 256:
         wanted = -(-(768 if M > 48 else 512) // groups)

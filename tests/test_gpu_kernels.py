@@ -114,7 +114,7 @@ def test_gemm_skinny(M, N, K_):
         assert torch.equal(one[0], out32[M - 1])
 
 
-@pytest.mark.parametrize("M", [1, 8, 17, 40, 64])
+@pytest.mark.parametrize("M", [1, 8, 12, 17, 40, 64])
 @pytest.mark.parametrize("N,K_,ranges", [(1536, 1536, 4), (1536, 8960, 5), (200, 72, 1), (72, 200, 1), (3584, 512, 2),
                                           (8192, 1024, 3)])
 def test_a_norm_folded_into_the_products_around_it(M, N, K_, ranges):
@@ -183,7 +183,7 @@ def test_embedding_rows(dtype):
     assert torch.allclose(stats[:, -1].cpu(), want[:, 192:].pow(2).sum(1), rtol=1e-5)  # the last, short tile
 
 
-@pytest.mark.parametrize("M", [17, 40, 64])
+@pytest.mark.parametrize("M", [9, 16, 17, 40, 64])
 @pytest.mark.parametrize("N,K_", [(32777, 264), (9000, 1024), (151936, 72)])
 def test_gemm_many_weight_rows(M, N, K_):
     """More than 16 rows of activations and many weight rows take the kernel that shares the
@@ -261,7 +261,7 @@ def test_gemm_partial_sums_on_small_workgroups(M):
     assert (parts[0].double().cpu() - first).abs().max() <= 2e-5 * float(want.abs().max())
 
 
-@pytest.mark.parametrize("M", [1, 8, 33, 64])
+@pytest.mark.parametrize("M", [1, 8, 13, 33, 64])
 @pytest.mark.parametrize("inter,K_", [(8960, 1536), (176, 64), (48, 72), (40, 72), (37888, 136)])
 def test_gemm_skinny_gated(M, inter, K_):
     torch.manual_seed(inter)
