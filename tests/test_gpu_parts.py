@@ -2,8 +2,9 @@
 mixer with state of its own, a toy mixer that caches one tensor of its own shape per token, a toy
 position encoding (which only encodes: it never sees a cache) and a toy architecture whose
 schedule names a layer twice, lets a stop read another stop's cache and scales its embedding and
-its logits are registered here, built and stepped (in portions, several sequences at once)
-without touching the framework's files."""
+its logits, and a toy norm and a toy arrangement of a layer's parts beside the built-in ones are
+registered here, built and stepped (in portions, several sequences at once) without touching the
+framework's files."""
 
 import math
 
@@ -444,3 +445,161 @@ def test_toy_mixer_with_one_cached_tensor_per_token(dtype):
             cache.release_passed(seq)
         cache.free_sequence(seq)
     assert cache.free_blocks() == (6,) and used == set(range(6))
+
+
+# ------------------------------------------------------------------ a norm and a block arrangement of the test's own
+@P.register_norm("toy_center")
+class CenterNorm(P.Part):
+    """y = w * (x - mean(x)) / sqrt(var(x) + eps): a norm that subtracts the mean (a test part, written
+    with library calls).  It has no `folded()`, so the products around it must hand over plain outputs
+    even in steps of a few rows, where an RMS norm would be carried by them."""
+
+    def tensors(self, prefix):
+        return {prefix + "weight": (self.spec.size,)}
+
+    def bind(self, prefix, weights):
+        self.weight = weights[prefix + "weight"].to(device=self.device, dtype=torch.float32)
+
+    def forward(self, stream, rows=None):
+        pending = stream.pending
+        delta = None if pending is None else (pending.sum(0) if pending.dim() == 3 else pending.float())
+        if rows is None:
+            stream.owed = stream.owed_to = None  # rows prepared for another norm are of no use here
+            if delta is not None:
+                stream.residual += delta
+                stream.pending = None
+            x = stream.residual
+        else:  # some rows only: the stream stays as it is
+            x = (stream.residual if delta is None else stream.residual + delta)[rows.long()]
+        centred = x - x.mean(-1, keepdim=True)
+        y = centred * torch.rsqrt(centred.pow(2).mean(-1, keepdim=True) + self.spec.eps) * self.weight
+        return y.to(self.dtype)
+
+
+@P.register_block("toy_parallel")
+class ParallelBlock:
+    """h = h + mixer(norm(h)) + feed_forward(norm(h)): both branches read the same normalised rows
+    and the layer has one norm.  Both outputs are left pending as two float32 terms for the next
+    norm to add; no branch is offered a sink."""
+
+    def __init__(self, layer_spec, dtype, device):
+        self.spec = layer_spec
+        self.mixer_norm = P.build_part(P.NORMS, "norm", layer_spec.mixer_norm, dtype, device)
+        self.mixer = P.build_part(P.MIXERS, "mixer", layer_spec.mixer, dtype, device)
+        self.feed_forward = P.build_part(P.FEED_FORWARDS, "feed-forward", layer_spec.feed_forward, dtype, device)
+
+    graph_safe = False
+    graph_max_rows = None
+
+    def _named(self):
+        s = self.spec
+        return ((self.mixer_norm, s.prefix + s.mixer_norm_prefix), (self.mixer, s.prefix + s.mixer_prefix),
+                (self.feed_forward, s.prefix + s.feed_forward_prefix))
+
+    def parts(self):
+        return [part for part, _ in self._named()]
+
+    def tensors(self):
+        out = {}
+        for part, prefix in self._named():
+            out.update(part.tensors(prefix))
+        return out
+
+    def bind(self, weights):
+        for part, prefix in self._named():
+            part.bind(prefix, weights)
+
+    def forward(self, ctx, stream):
+        x = P.plain_rows(self.mixer_norm.forward(stream))
+        ctx.sink = None
+        terms = []
+        for part in (self.mixer, self.feed_forward):
+            y = part.forward(ctx, x)
+            terms.append(y.sum(0) if y.dim() == 3 else y.float())
+        stream.pending = torch.stack(terms)
+
+
+class ParallelToyConfig:
+    """Two layers: a parallel block around the centring norm, then the ordinary block with RMS norms;
+    the final norm centres again."""
+
+    def __init__(self, cfg):
+        self.cfg = dict(cfg)
+
+    def to_json_dict(self):
+        return dict(self.cfg)
+
+    def plan(self):
+        c = self.cfg
+        H, hd = c["hidden_size"], c["head_dim"]
+        centre = NormSpec(size=H, eps=c["eps"], kind="toy_center")
+        rms = NormSpec(size=H, eps=c["eps"])
+        attn = MixerSpec(hidden_size=H, num_heads=c["heads"], num_kv_heads=c["kv_heads"], head_dim=hd,
+                         scale=hd ** -0.5, qkv_bias=True, position=PositionSpec(rotary_dim=hd, theta=c["theta"]))
+        ffn = FeedForwardSpec(hidden_size=H, intermediate_size=c["inter"])
+        layers = (LayerSpec("model.layers.0.", attn, ffn, centre, centre, arrangement="toy_parallel"),
+                  LayerSpec("model.layers.1.", attn, ffn, rms, rms))
+        return ModelPlan("ParallelToyForCausalLM", H, c["vocab"], layers, (ScheduleEntry(0), ScheduleEntry(1)), centre,
+                         "model.embed_tokens.weight", "lm_head.weight", "model.norm.")
+
+
+pae.register_architecture("ParallelToyForCausalLM", ParallelToyConfig)
+PARALLEL_TOY = dict(architectures=["ParallelToyForCausalLM"], hidden_size=64, head_dim=16, heads=4, kv_heads=2, inter=80,
+                    vocab=131, eps=1e-5, theta=10000.0)
+
+
+def parallel_toy_plain_logits(w, c, ids):
+    """The architecture above written out plainly (float64, whole sequence, no cache)."""
+    w = {k: v.double() for k, v in w.items()}
+    cfg = dict(num_attention_heads=c["heads"], num_key_value_heads=c["kv_heads"], head_dim=c["head_dim"],
+               hidden_size=c["hidden_size"], rope_theta=c["theta"])
+    pos = torch.arange(len(ids))
+
+    def centre(x, weight):
+        d = x - x.mean(-1, keepdim=True)
+        return d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + c["eps"]) * weight
+
+    x = w["model.embed_tokens.weight"][ids]
+    h = centre(x, w["model.layers.0.input_layernorm.weight"])
+    x = x + plain.self_attention(w, "model.layers.0.", cfg, h, pos, None) + plain.swiglu_mlp(w, "model.layers.0.", h)
+    h = plain.rms_norm(x, w["model.layers.1.input_layernorm.weight"], c["eps"])
+    x = x + plain.self_attention(w, "model.layers.1.", cfg, h, pos, None)
+    h = plain.rms_norm(x, w["model.layers.1.post_attention_layernorm.weight"], c["eps"])
+    x = x + plain.swiglu_mlp(w, "model.layers.1.", h)
+    return plain.linear(centre(x, w["model.norm.weight"]), w["lm_head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_norm_and_block_arrangement_are_registered_built_and_stepped(tmp_path, dtype):
+    """A norm and an arrangement of a layer's parts defined in this file, beside the built-in ones in
+    the same model: portions of prompts, single tokens (where the built-in norms are carried by the
+    products around them and the toy norm is not) and both together."""
+    assert "toy_parallel" in P.BLOCKS and "toy_center" in P.NORMS
+    config = pae.read_config_dict(PARALLEL_TOY)
+    folder = pae.write_model_folder(config, 8, str(tmp_path / "parallel_toy"), std=0.08, norm_std=0.1)
+    model = pae.load_model(folder, dtype)
+    names = model.expected_tensors()
+    assert "model.layers.0.input_layernorm.weight" in names
+    assert "model.layers.0.post_attention_layernorm.weight" not in names  # the parallel block has one norm
+    assert not model.graph_safe
+    cache = model.new_cache(16, 12, 3)
+    runner = pae.StepRunner(model, cache)
+    w = {k: v.float() for k, v in pae.load_weights(folder, names).items()}
+    gen = torch.Generator().manual_seed(4)
+    seqs = {s: torch.randint(0, 131, (n,), generator=gen).tolist() for s, n in ((0, 40), (1, 23), (2, 9))}
+    want = {s: parallel_toy_plain_logits(w, PARALLEL_TOY, ids).float() for s, ids in seqs.items()}
+    tol = helpers_tol(dtype, max(float(v.abs().max()) for v in want.values()))
+    done = {s: 0 for s in seqs}
+    for s in seqs:
+        assert cache.create_sequence(s)
+    plans = ([(0, 30), (1, 20)], [(0, 1), (1, 1), (2, 7)], [(0, 1), (1, 1), (2, 1)], [(0, 1), (1, 1), (2, 1)], [(0, 7)])
+    for plan in plans:
+        entries = []
+        for s, n in plan:
+            cache.reserve(s, n)
+            entries.append(pae.StepEntry(s, tuple(seqs[s][done[s]:done[s] + n]), tuple(range(n))))
+        got = runner.run(entries).cpu()
+        ref = torch.cat([want[s][done[s]:done[s] + n] for s, n in plan])
+        assert float((got - ref).abs().max()) <= tol, plan
+        for s, n in plan:
+            done[s] += n
