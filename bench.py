@@ -69,6 +69,10 @@ class Unresolved(RuntimeError):
     """The passes of a measurement disagree by more than the limit: no figure is given."""
 
 
+class Refused(RuntimeError):
+    """The run that was asked for cannot be made at this shape; the message says why."""
+
+
 def settle(passes):
     """(median, range) of the passes' times."""
     ordered = sorted(passes)
@@ -140,6 +144,12 @@ def decode_run(model, cfg, batch: int, ctx: int, steps: int, warmup: int, block_
     prompt_len = ctx - warmup // 2 - 1
     slack = batch * prompt_len // 2048 + 4
     max_new = warmup + ESCALATED_PASSES * steps + slack + 2
+    limit = cfg.get("max_position_embeddings")
+    if prompt_len < 1 or (limit and prompt_len + max_new > limit):
+        raise Refused(f"a context of {ctx} tokens with {max_new} new tokens to decode on top (warm-up, up to "
+                      f"{ESCALATED_PASSES} passes of {steps} steps and slack) runs past the shape's "
+                      f"max_position_embeddings of {limit}: the scheduler would reject the requests; ask for a "
+                      f"context of at most {limit - max_new + warmup // 2 + 1}")
     blocks = batch * (-(-(prompt_len + max_new) // block_size) + 1) + 2
     dtype = "bfloat16" if model.dtype == torch.bfloat16 else "float32"
     engine = pae.Engine(model, dtype=dtype, block_size=block_size, num_blocks=blocks, max_num_seqs=batch,
@@ -178,6 +188,50 @@ def decode_run(model, cfg, batch: int, ctx: int, steps: int, warmup: int, block_
     del engine, sched
     torch.cuda.empty_cache()
     return median, spread, sum(held) / len(held), blocks, recordings
+
+
+def baseline_decode_run(model, cfg, batch: int, prompt_len: int = 512, new_tokens: int = 256, block_size: int = 16):
+    """The reference's own decode workload: `batch` requests of `prompt_len`-token prompts, `new_tokens`
+    greedy tokens each.  The prompts run first, untimed (each yields its request's first token); the clock
+    runs over the decode steps that give the other new_tokens - 1 tokens of every request, to the last
+    token's arrival on the host.  One engine serves all passes (its recorded steps are made in the first
+    pass, which is discarded).  Returns (median seconds, range, decoded tokens a pass, mean tokens held)."""
+    import torch
+    import paged_attention_engine_amd as pae
+
+    dtype = "bfloat16" if model.dtype == torch.bfloat16 else "float32"
+    blocks = batch * (-(-(prompt_len + new_tokens) // block_size) + 1) + 2
+    engine = pae.Engine(model, dtype=dtype, block_size=block_size, num_blocks=blocks, max_num_seqs=batch,
+                        max_num_batched_tokens=2048)
+    sched = engine.scheduler
+    gen = torch.Generator().manual_seed(DECODE_TOKEN_SEED)
+    counted, number = [], [0]
+
+    def one_pass():
+        number[0] += 1
+        names = [f"p{number[0]}b{b}" for b in range(batch)]
+        for name in names:
+            prompt = torch.randint(0, cfg["vocab_size"], (prompt_len,), generator=gen).tolist()
+            assert engine.add_request(pae.Request(name, tuple(prompt), new_tokens))
+        while len(sched.waiting) or any(s.prefilling for s in sched.running):
+            engine.step()
+        before = sum(len(s.generated) for s in sched.running)
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        engine.run_to_completion()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - start
+        done = sum(len(engine.finished[name].generated) for name in names)
+        assert done == batch * new_tokens and not sched.running
+        counted.append(done - before)
+        return elapsed
+
+    one_pass()  # warm-up, discarded
+    median, spread, _ = measured(one_pass, f"{prompt_len}+{new_tokens} decode at batch {batch}")
+    assert len(set(counted)) == 1, counted  # every pass decodes the same number of tokens
+    del engine, sched
+    torch.cuda.empty_cache()
+    return median, spread, counted[0], batch * (prompt_len + new_tokens / 2)
 
 
 def prefill_run(model, cfg, T: int, block_size: int = 16):
@@ -240,6 +294,9 @@ def main() -> int:
 
     try:
         return report(args, cfg, elem, model)
+    except Refused as err:
+        print(f"bench.py: {err}")
+        return 2
     except Unresolved as err:
         print(json.dumps({"metric": f"decode tok/s at batch {args.batch}, context {args.ctx} ({args.shape_name})",
                           "value": None, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -282,11 +339,36 @@ def report(args, cfg, elem, model) -> int:
         record["prefill"] = {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
                              "frac": round(prefill_flops(cfg, T) / pre_s / PEAK_FLOPS[args.dtype], 4),
                              "range_ms": round(pre_range * 1e3, 3)}
-        points = {}
+        # tokens a second, and beside each the share of the HBM peak that its bytes a step come to
+        points, fracs = {}, {}
+        short = max(8, args.steps // 2)
+
+        def point(name, cfg_, batch, step_seconds, tokens_held):
+            points[name] = round(batch / step_seconds, 2)
+            moved = weight_bytes(cfg_, elem) + kv_bytes(cfg_, tokens_held, elem)
+            fracs[name] = round(moved / step_seconds / 1e9 / HBM_PEAK_GBS, 4)
+
         for b in (1, 64):
-            s, _, _, _, _ = decode_run(model, cfg, b, args.ctx, max(8, args.steps // 2), 4)
-            points[f"decode_b{b}"] = round(b / s, 2)
+            s, _, held, _, _ = decode_run(model, cfg, b, args.ctx, short, 4)
+            point(f"decode_b{b}", cfg, b, s, held)
+        if args.model == "1.5b" and args.layers == args.full_layers and args.ctx == 4096:
+            # the reference's own decode workload: 512-token prompts, 256 greedy tokens each
+            for b in (1, 8, 64):
+                s, _, decoded, held = baseline_decode_run(model, cfg, b)
+                point(f"decode_512p256_b{b}", cfg, b, s / (decoded / b), held)
+            # a longer context at the headline batch
+            s, _, held, _, _ = decode_run(model, cfg, 8, 16384, short, 4)
+            point("decode_b8_ctx16384", cfg, 8, s, held)
+            # the 7B layer sizes at the headline batch and context
+            import torch
+            del model
+            torch.cuda.empty_cache()
+            cfg7 = dict(OTHER_SHAPES["7b"])
+            model = build_model(cfg7, args.dtype)
+            s, _, held, _, _ = decode_run(model, cfg7, 8, 4096, short, 4)
+            point("decode_7b_b8", cfg7, 8, s, held)
         record["points"] = points
+        record["points_hbm_frac"] = fracs
     record["provenance"] = provenance(model, {"pool_pages": pages, "graph_recordings_in_run": recordings})
     print(json.dumps(record))
     return 0

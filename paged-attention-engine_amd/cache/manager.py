@@ -31,6 +31,7 @@ live there, where no sequence's data ever is.
 from __future__ import annotations
 
 from dataclasses import dataclass
+from collections import deque
 from typing import Dict, List, Mapping, Optional, Sequence, Tuple, Union
 
 import torch
@@ -122,7 +123,7 @@ class StateSlots:
 
     def __init__(self, num_slots: int) -> None:
         self.num_slots = num_slots
-        self._free = list(range(num_slots))
+        self._free = deque(range(num_slots))
         self._held: Dict[int, int] = {}
 
     @property
@@ -134,7 +135,7 @@ class StateSlots:
             raise KeyError(f"sequence {seq_id} already holds a state slot")
         if not self._free:
             return None
-        slot = self._free.pop(0)
+        slot = self._free.popleft()
         self._held[seq_id] = slot
         return slot
 
@@ -207,12 +208,6 @@ class CacheManager:
         """The cached tensors of a stop by name, each [block][*page shape]."""
         g, i = self._group_of_entry[entry]
         return {name: pool[i] for name, pool in self.groups[g].pools.items()}
-
-    def kv_of(self, entry: int) -> Tuple[torch.Tensor, torch.Tensor]:
-        """(keys, values) of a stop whose mixer declared `attention_pages`: keys
-        [block][kv head][block_size][head_dim], values [block][kv head][head_dim][block_size]."""
-        pages = self.pages_of(entry)
-        return pages["k"], pages["v"]
 
     def state_of(self, entry: int) -> torch.Tensor:
         return self.state_tensors[entry]

@@ -32,7 +32,7 @@ class EngineConfig:
     admission_margin_blocks: int = ADMISSION_MARGIN_BLOCKS
     max_num_seqs: Optional[int] = None
     max_num_batched_tokens: Optional[int] = None
-    num_state_slots: Optional[int] = None  # default: max_num_seqs, else 64
+    num_state_slots: Optional[int] = None  # default: max_num_seqs; else see `state_slots_for`
     device: str = "cuda:0"
 
     def __post_init__(self) -> None:
@@ -71,8 +71,16 @@ class EngineConfig:
             raise ValueError(f"the cache's budget does not pay for one page of {page_bytes} bytes in every group")
         return count
 
-    @property
-    def state_slots(self) -> int:
+    def state_slots_for(self, pages: int, keeps_state: bool) -> int:
+        """Slots for per-request state, which also bound the live sequences: as given, else
+        `max_num_seqs`.  With neither, a model that keeps no such state gets one slot per page (a live
+        sequence holds at least a page, so the slots never bind); a model that does keep state has its
+        slots allocated up front, and the caller must say how many."""
         if self.num_state_slots is not None:
             return self.num_state_slots
-        return self.max_num_seqs if self.max_num_seqs is not None else 64
+        if self.max_num_seqs is not None:
+            return self.max_num_seqs
+        if keeps_state:
+            raise ValueError("this model keeps per-request state in slots that are allocated up front: "
+                             "give max_num_seqs or num_state_slots")
+        return max(1, pages)

@@ -33,6 +33,7 @@ class NormSpec(PartSpec):
     size: int = 0
     eps: float = 0.0
     kind: str = "rmsnorm"
+    weight_name: str = "weight"  # the tensor's name below the norm's prefix
 
 
 @dataclass(frozen=True)
@@ -62,6 +63,12 @@ class MixerSpec(PartSpec):
     window: Optional[int] = None
     position: Optional[PositionSpec] = None
     kind: str = "attention"
+    # names of the four projections below the mixer's prefix (each with ".weight" and, where the
+    # spec says so, ".bias"): an architecture that calls them otherwise sets these, not a new mixer
+    q_name: str = "q_proj"
+    k_name: str = "k_proj"
+    v_name: str = "v_proj"
+    o_name: str = "o_proj"
 
 
 @dataclass(frozen=True)
@@ -70,6 +77,10 @@ class FeedForwardSpec(PartSpec):
     intermediate_size: int = 0
     activation: str = "silu"
     kind: str = "swiglu"
+    # names of the three projections below the feed-forward's prefix
+    gate_name: str = "gate_proj"
+    up_name: str = "up_proj"
+    down_name: str = "down_proj"
 
 
 @dataclass(frozen=True)
@@ -114,6 +125,9 @@ class ModelPlan:
     head_name: Optional[str]  # None: the head shares the embedding matrix
     final_norm_prefix: str
     max_positions: Optional[int] = None
+    # tensors a checkpoint of this architecture may hold without the model using them (a head stored
+    # although it is tied to the embedding, say): the loader passes over them
+    optional_names: Tuple[str, ...] = ()
     # what some architectures do around the blocks (the reference's model does none of it:
     # engine/model.py:401,453-455 gathers rows and multiplies by the head as they are)
     embedding_scale: float = 1.0            # the gathered rows are multiplied by this

@@ -65,14 +65,18 @@ int pae_sample(int* tokens, const float* logits, int64_t ld, const float* temper
 // under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
 // counterpart in the reference.  The chunk results live in a buffer that is part of the library's
 // image on every GPU (16 bytes a slot, PAE_SAMPLE_STATIC_SLOTS slots = 512 KiB, held by each GPU
-// the library runs on until the process ends); its device address is looked up once per device at
-// the first call there.  num_rows * pae_sample_chunks(vocab) beyond the slots is refused.  The call
+// the library runs on until the process ends); its device address is looked up once per device, for
+// the device that `stream` belongs to (the current device for the null stream), at the first call
+// there or by pae_sample_static_prepare() with that device current.  That first lookup asks the
+// runtime and must not fall inside a stream capture (it is refused there): prepare, or call once,
+// before capturing.  num_rows * pae_sample_chunks(vocab) beyond the slots is refused.  The call
 // itself calls no hipMalloc, hipFree or other allocating routine.  Every call on a GPU uses that
 // GPU's one buffer: calls that overlap on one GPU (several streams or threads) race, so issue them
 // one after the other.  Nothing in the buffer needs clearing between calls: a call writes every
 // slot before it reads it.  Same results as pae_sample, bit for bit.
 #define PAE_SAMPLE_STATIC_SLOTS 32768
 int pae_sample_static_slots();
+int pae_sample_static_prepare();
 int pae_sample_static(int* tokens, const float* logits, int64_t ld, const float* temperature,
                       const float* uniform, int num_rows, int vocab, hipStream_t stream);
 }

@@ -1,0 +1,675 @@
+// A decode step's layers as one resident kernel.
+//
+// A step in which every sequence brings one token is a chain of short dependent kernels: per
+// layer the query/key/value product, the split attention and its merge, the output product, the
+// gated product and the down product.  Each of them moves a few megabytes and costs 4 to 7 us
+// however little it moves, because a kernel boundary drains the chip and the next kernel's first
+// loads wait out the memory's latency.  Here the chain is a list of phases that one kernel walks:
+// as many workgroups as compute units stay resident for the whole step (1,024 threads each, four
+// "quads" of four wavefronts) and meet at a barrier of their own between phases.
+//
+// Phases are the existing kernels' work, cut into items that the quads take in turn:
+//   product    one item = 16 weight rows x one k range, the quad's wavefronts taking 32-wide k
+//              steps in turn exactly as gemm_skinny_kernel<1, 1, EPI, 4> does (the same sums in the
+//              same order, bit for bit), k ranges added up by ticket, any of that kernel's epilogues;
+//   attention  one item = (token, key/value head, split of 128 keys) as attn_decode_kernel; the quad
+//              that draws a (token, head)'s last ticket merges its splits, four groups of splits as
+//              attn_decode_merge_kernel has them.
+//
+// What one workgroup writes and another reads after the barrier is written through to the memory
+// side with device-scope stores (the dies' L2s are not coherent with one another, see
+// skinny_device.h), acknowledged before the workgroup arrives at the barrier, and every wavefront
+// invalidates its caches after the barrier before it reads.  Every wait is bounded: a workgroup
+// that has polled `spin_limit` times gives up, leaves an error code for the host and for the other
+// workgroups, and the kernel ends.
+#include "common.h"
+#include "api.h"
+#include "skinny_device.h"
+#include "attention_device.h"
+
+#define PROG_PRODUCT 1
+#define PROG_ATTENTION 2
+#ifndef PROG_QUADS
+#define PROG_QUADS 2
+#endif
+#define PROG_THREADS (PROG_QUADS * 4 * PAE_WAVE)
+#define PROG_MAX_ROWS 16
+#define PROG_SPLIT 128    // keys per split of the attention phase: pae_attn_decode_split()
+#define PROG_MERGE_ITEMS 256  // (heads of a group) x (head_dim / 4) that one quad merges
+
+struct ProgPhase {
+  int type, epilogue;
+  // product: out[M, N] (+)= A[M, K] W[N, K]^T through the epilogue
+  int M, N, K, splits, k_per_split, b_is_f32;
+  const bf16_t* W;
+  const void* bias;
+  const bf16_t* A;
+  void* out;
+  int64_t lda, ldc;
+  SkinnyNorm norm;
+  SkinnyRope rope;
+  float* ticket_parts;
+  int* ticket_counters;
+  // decode attention
+  const int4* dec_work;
+  const int* block_tables;
+  const bf16_t* q;
+  bf16_t* attn_out;
+  const bf16_t* k_cache;
+  const bf16_t* v_cache;
+  float* part_acc;
+  float* part_ml;
+  int64_t q_stride, out_stride;
+  int num_dec, max_splits, max_blocks, bs, nh, nkv, hd, window;
+  float scale_log2;
+  int pad_[3];
+};
+static_assert(sizeof(ProgPhase) % 16 == 0, "phases are copied as 16-byte pieces");
+
+// A barrier across the workgroups in two levels.  Arrivals are counted in one counter per die (the
+// workgroup's number mod 8; each in a 128-byte line of its own: arrivals at one address are taken one
+// after the other, about 15 ns each, and are 32 this way, not 256); the last arrival of a die counts
+// once at the top, and the last of those publishes the barrier's number, which everybody polls.  (All
+// workgroups polling the eight counters themselves, with arrivals that nobody waits for, is slower at
+// 256 workgroups, 4.7 against 4.0 us a phase: the polls queue up in front of the arrivals.)  The
+// counters only ever grow (barrier number e is complete when a counter stands at e times its members),
+// so nothing is put back and nothing orders a reset against the next arrival.  One such block serves
+// one grid size.
+struct ProgBarrier {
+  unsigned die[8][32];
+  unsigned top[32];
+  unsigned done[32];   // [0] number of the last complete barrier
+  unsigned error[32];  // [0] 0, or 1 + the phase after which a workgroup gave up
+};
+
+__device__ __forceinline__ unsigned barrier_members(unsigned die) { return (gridDim.x - die + 7) / 8; }
+
+// Barriers completed before this launch, as the workgroup's own die counter tells (it cannot pass the
+// next multiple of its members before this workgroup has arrived).
+__device__ __forceinline__ unsigned barrier_epoch_at_start(const ProgBarrier* bar) {
+  const unsigned die = blockIdx.x % 8;
+  return __hip_atomic_load(&bar->die[die][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) / barrier_members(die);
+}
+
+// True when every workgroup has arrived and the caches are clean; false when the program is dead
+// (this workgroup or another gave up), in which case the kernel must end.  `epoch` lives in thread 0.
+__device__ __forceinline__ bool grid_barrier(ProgBarrier* bar, unsigned& epoch, int* s_dead, int spin_limit, int phase) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's written-through stores have arrived
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    epoch += 1;
+    const unsigned die = blockIdx.x % 8, dies = gridDim.x < 8 ? gridDim.x : 8;
+    const unsigned arrived = __hip_atomic_fetch_add(&bar->die[die][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (arrived + 1 == barrier_members(die) * epoch) {
+      const unsigned up = __hip_atomic_fetch_add(&bar->top[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (up + 1 == dies * epoch) __hip_atomic_store(&bar->done[0], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    int spins = 0;
+    bool alive = true;
+    while ((int)(__hip_atomic_load(&bar->done[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
+      if (++spins > spin_limit ||
+          (spins % 64 == 0 && __hip_atomic_load(&bar->error[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+        alive = false;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (!alive) {
+      __hip_atomic_store(&bar->error[0], (unsigned)(phase + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *s_dead = 1;
+    }
+    // Nothing read below may come from a stale cache line: the compute unit's vector cache and the
+    // die's L2 drop what they hold of memory that other dies may have written.  Once a workgroup is
+    // enough (its wavefronts share the caches); every wavefront doing it costs 30 us a barrier.
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
+  __syncthreads();
+  return *s_dead == 0;
+}
+
+// ---------------------------------------------------------------------------------------- product
+// Item i of a product phase is tile i % tiles of 16 weight rows over k range i / tiles; quad q of
+// workgroup b takes the items base + q * gridDim.x + b of every round.  The quad's four wavefronts
+// take the 32-wide k steps of the range in turn and their sums are added in wavefront order through
+// LDS (two buffers that take turns, so that a round needs one workgroup barrier).
+//
+// A quad asks for the first fragments of its coming item while the current one finishes: the weights
+// and activations of the next round's item, or, at the end of the phase, the weights of its first item
+// of the next phase (weights do not depend on what the barrier waits for; activations do, and are
+// asked for behind it).  `Ahead` carries them from item to item and from phase to phase.
+#define PROG_U 4  // k steps of a wavefront whose loads are in flight together, as in gemm_skinny_kernel<1, 1, EPI, 4>
+struct Ahead {
+  bf16x8 wf[PROG_U], af[PROG_U];
+  bool has_w, has_a;  // the same in every lane
+};
+
+struct ItemPlace {
+  const bf16_t* wrow;  // this lane's weight row (lane / 4 of the tile, through the rotation's row order if any)
+  int tile, split, k_lo, k_hi;
+};
+
+__device__ __forceinline__ ItemPlace place_of(const ProgPhase& ph, int item) {
+  const int lane = threadIdx.x % PAE_WAVE, lrow = lane / 4;
+  const int tiles = (ph.N + 15) / 16;
+  ItemPlace at;
+  at.tile = item % tiles;
+  at.split = item / tiles;
+  at.k_lo = at.split * ph.k_per_split;
+  at.k_hi = min(ph.K, at.k_lo + ph.k_per_split);
+  int n = 16 * at.tile + lrow;
+  if (ph.epilogue == EPI_ROPE) {
+    const int per_head = ph.rope.hd / 16;
+    n = at.tile / per_head * ph.rope.hd + rope_feature(at.tile % per_head, lrow, ph.rope.rot);
+  }
+  at.wrow = ph.W + (int64_t)(n < ph.N ? n : ph.N - 1) * ph.K;  // rows past N are loaded from the last row and never stored
+  return at;
+}
+
+// The fragments of the PROG_U steps from `kb` on of a row (loads are unconditional, from clamped addresses).
+__device__ __forceinline__ void ask_row(bf16x8 (&frag)[PROG_U], const bf16_t* row, int kb, int K) {
+  const int lkg = threadIdx.x % 4;
+#pragma unroll
+  for (int u = 0; u < PROG_U; ++u) {
+    const int k = kb + 128 * u + 8 * lkg;
+    frag[u] = *reinterpret_cast<const bf16x8*>(row + (k < K - 8 ? k : K - 8));
+  }
+}
+
+__device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPhase* next, float* quad_lds, int& parity,
+                                              Ahead& ahead) {
+  const int lane = threadIdx.x % PAE_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE), quad = wave / 4, wq = wave % 4;
+  const int M = ph.M, N = ph.N, K = ph.K;
+  const int tiles = (N + 15) / 16, items = tiles * ph.splits, per_round = gridDim.x * PROG_QUADS;
+  const int lrow = lane / 4, g4 = lane / 16;
+  const int fetch_from = ((lane % 16) * 4 + lane / 16) * 4;
+  constexpr int U = PROG_U, KW = 128, STEP = KW * U;
+  float scale[1] = {1.0f};
+  if (wq == 0) row_scales<1>(scale, ph.norm, M, K);  // asked for at once: the shares arrive while the products run
+  const bf16_t* arow = ph.A + (int64_t)(lrow < M ? lrow : M - 1) * ph.lda;
+  const bf16x8 zero = {};
+  struct Batch {
+    bf16x8 wf[U], af[U];
+  };
+  const int first = quad * gridDim.x + blockIdx.x;
+  for (int base = 0; base < items; base += per_round) {
+    const int item = base + first;
+    const bool live = item < items;  // the same in every lane of the quad
+    f32x4 acc[1][1] = {{(f32x4){0.f, 0.f, 0.f, 0.f}}};
+    ItemPlace at = {};
+    if (live) {
+      at = place_of(ph, item);
+      const int k_hi = at.k_hi;
+      auto load = [&](Batch& b, int kb) {
+        ask_row(b.wf, at.wrow, kb, K);
+        ask_row(b.af, arow, kb, K);
+      };
+      auto multiply = [&](Batch& b, int kb) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const bool kok = kb + KW * u + 8 * g4 < k_hi;
+          const bf16x8 a = to_mfma_order(b.af[u], fetch_from);
+          const bf16x8 moved = to_mfma_order(b.wf[u], fetch_from);
+          acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kok ? moved : zero, a, acc[0][0], 0, 0, 0);
+        }
+      };
+      int kb = at.k_lo + 32 * wq;
+      Batch b0, b1;
+      if (kb < k_hi) {
+        if (ahead.has_w) {
+#pragma unroll
+          for (int u = 0; u < U; ++u) b0.wf[u] = ahead.wf[u];
+        } else {
+          ask_row(b0.wf, at.wrow, kb, K);
+        }
+        if (ahead.has_a) {
+#pragma unroll
+          for (int u = 0; u < U; ++u) b0.af[u] = ahead.af[u];
+        } else {
+          ask_row(b0.af, arow, kb, K);
+        }
+      }
+      ahead.has_w = ahead.has_a = false;
+      // the coming round's item, asked for as soon as this item's last loads are out
+      bool asked = false;
+      auto ask_ahead = [&]() {
+        asked = true;
+        if (item + per_round < items) {
+          const ItemPlace then = place_of(ph, item + per_round);
+          ask_row(ahead.wf, then.wrow, then.k_lo + 32 * wq, K);
+          ask_row(ahead.af, arow, then.k_lo + 32 * wq, K);
+          ahead.has_w = ahead.has_a = true;
+        }
+      };
+      while (kb < k_hi) {
+        if (kb + STEP < k_hi) load(b1, kb + STEP);
+        else if (!asked) ask_ahead();
+        multiply(b0, kb);
+        kb += STEP;
+        if (kb >= k_hi) break;
+        if (kb + STEP < k_hi) load(b0, kb + STEP);
+        else if (!asked) ask_ahead();
+        multiply(b1, kb);
+        kb += STEP;
+      }
+      if (!asked) ask_ahead();
+    }
+    float* s_part = quad_lds + parity * (3 * 4 * PAE_WAVE);  // [3][4][64]
+    parity ^= 1;
+    if (live && wq > 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s_part[((wq - 1) * 4 + i) * PAE_WAVE + lane] = acc[0][0][i];
+    }
+    __syncthreads();
+    if (!live || wq > 0) continue;
+#pragma unroll
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[0][0][i] += s_part[(w * 4 + i) * PAE_WAVE + lane];
+    if (ph.epilogue != EPI_F32 && ph.splits > 1) {
+      f32x4 mine[1] = {acc[0][0]};
+      if (!add_up_k_ranges<1>(mine, at.tile, at.split, ph.splits, SkinnyTickets{ph.ticket_parts, ph.ticket_counters})) continue;
+      acc[0][0] = mine[0];
+    }
+#define PROG_EPILOGUE(EPI)                                                                                          \
+  skinny_epilogue<1, 1, EPI, true>(acc, at.tile, -1, ph.out, ph.ldc, ph.bias, ph.b_is_f32, M, N, at.split, (int64_t)M * N, \
+                                   ph.rope, ph.norm, scale)
+    switch (ph.epilogue) {  // the one place where the epilogues part ways: the products above are the same code for all
+      case EPI_BF16: PROG_EPILOGUE(EPI_BF16); break;
+      case EPI_F32: PROG_EPILOGUE(EPI_F32); break;
+      case EPI_SWIGLU: PROG_EPILOGUE(EPI_SWIGLU); break;
+      case EPI_ROPE: PROG_EPILOGUE(EPI_ROPE); break;
+      default: PROG_EPILOGUE(EPI_RESIDUAL); break;
+    }
+#undef PROG_EPILOGUE
+  }
+  // the weights of this quad's first item of the next phase, on their way while the barrier is crossed
+  if (!ahead.has_w && next && next->type == PROG_PRODUCT && first < (next->N + 15) / 16 * next->splits) {
+    const ItemPlace then = place_of(*next, first);
+    ask_row(ahead.wf, then.wrow, then.k_lo + 32 * wq, next->K);
+    ahead.has_w = true;
+  }
+}
+
+// -------------------------------------------------------------------------------------- attention
+// Item i is split i % max_splits of key/value head (i / max_splits) % nkv of token i / (max_splits *
+// nkv); items whose split lies outside the token's keys are empty.  Inside an item the quad is
+// attn_decode_kernel's workgroup; it then leaves its partial result in memory and draws a ticket
+// from the (token, head)'s counter, and the quad that draws the last one merges all of the splits:
+// its four wavefronts are attn_decode_merge_kernel's four groups of splits.
+template <int HD>
+__device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad_lds, int* s_flag) {
+  constexpr int TPW = PROG_SPLIT / 64, ROWS = HD / 4 + 2;
+  const int lane = threadIdx.x % PAE_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE), quad = wave / 4, wq = wave % 4;
+  const int col = lane % 16, g4 = lane / 16;
+  const int nkv = ph.nkv, g = ph.nh / nkv, bs = ph.bs, window = ph.window, max_splits = ph.max_splits;
+  const int items = ph.num_dec * nkv * max_splits, per_round = gridDim.x * PROG_QUADS;
+  const int page_elems = bs * HD;
+  const int merge_items = g * (HD / 4);
+  for (int base = 0; base < items; base += per_round) {
+    const int item = base + quad * gridDim.x + blockIdx.x;
+    bool live = item < items;
+    const int split = live ? item % max_splits : 0, kvh = live ? item / max_splits % nkv : 0;
+    const int tok_index = live ? item / (max_splits * nkv) : 0;
+    const int4 work = ph.dec_work[tok_index];
+    const int pos[1] = {work.y};
+    const int start[1] = {(window > 0 && pos[0] - window + 1 > 0) ? pos[0] - window + 1 : 0};
+    const int s_first = start[0] / PROG_SPLIT, s_last = pos[0] / PROG_SPLIT;
+    live = live && split >= s_first && split <= s_last;
+    AttnState<HD, 1> st;
+    st.m[0] = NEG_BIG;
+    st.l[0] = 0.f;
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) st.acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    if (live) {
+      const int lo = max(split * PROG_SPLIT, start[0] / 16 * 16);
+      const int hi = min((split + 1) * PROG_SPLIT, pos[0] + 1);
+      const int* table = ph.block_tables + (int64_t)work.z * ph.max_blocks;
+      bf16x8 qf[1][HD / 32];
+      const bf16_t* qrow = ph.q + (int64_t)work.x * ph.q_stride + (int64_t)(kvh * g + (col < g ? col : 0)) * HD;
+#pragma unroll
+      for (int j = 0; j < HD / 32; ++j) {
+        qf[0][j] = *reinterpret_cast<const bf16x8*>(qrow + 32 * j + 8 * g4);
+        if (col >= g)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) qf[0][j][e] = (__bf16)0.f;
+      }
+      const int tile_lo = lo / 16, tile_hi = (hi + 15) / 16;
+      bf16x8 kf[TPW][HD / 32];
+      s16x4 vf[TPW][HD / 16];
+#pragma unroll
+      for (int j = 0; j < TPW; ++j) {  // a tile past the end is loaded from the first tile's place and not used
+        const int tile = tile_lo + wq + 4 * j;
+        const int key0 = (tile < tile_hi ? tile : tile_lo) * 16;
+        const int64_t at = ((int64_t)table[key0 / bs] * nkv + kvh) * page_elems;
+        load_kv_tile<HD>(kf[j], vf[j], ph.k_cache + at + (int64_t)(key0 % bs) * HD, ph.v_cache + at + key0 % bs, bs);
+      }
+#pragma unroll
+      for (int j = 0; j < TPW; ++j) {
+        const int tile = tile_lo + wq + 4 * j;
+        keys_to_mfma_order<HD>(kf[j]);
+        if (tile < tile_hi) attn_tile<HD, 1>(st, kf[j], vf[j], qf, tile * 16, pos, start, ph.scale_log2);
+      }
+      if (wq > 0) {
+        float* mine = quad_lds + (wq - 1) * ROWS * PAE_WAVE;
+#pragma unroll
+        for (int t = 0; t < HD / 16; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mine[(4 * t + i) * PAE_WAVE + lane] = st.acc[0][t][i];
+        mine[(HD / 4) * PAE_WAVE + lane] = st.m[0];
+        mine[(HD / 4 + 1) * PAE_WAVE + lane] = st.l[0];
+      }
+    }
+    __syncthreads();
+    int to_merge = -1;  // the (token, head) whose last ticket this quad drew
+    if (live && wq == 0) {
+#pragma unroll
+      for (int w = 0; w < 3; ++w) {
+        const float* theirs = quad_lds + w * ROWS * PAE_WAVE;
+        const float mw = theirs[(HD / 4) * PAE_WAVE + lane];
+        const float m_new = fmaxf(st.m[0], mw);
+        const float f0 = exp2f(st.m[0] - m_new), fw = exp2f(mw - m_new);
+#pragma unroll
+        for (int t = 0; t < HD / 16; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) st.acc[0][t][i] = st.acc[0][t][i] * f0 + theirs[(4 * t + i) * PAE_WAVE + lane] * fw;
+        st.l[0] = st.l[0] * f0 + theirs[(HD / 4 + 1) * PAE_WAVE + lane] * fw;
+        st.m[0] = m_new;
+      }
+      float l = st.l[0];
+      l += __shfl_xor(l, 16, PAE_WAVE);
+      l += __shfl_xor(l, 32, PAE_WAVE);
+      const int pair = tok_index * nkv + kvh;
+      if (col < g) {
+        const int64_t slot = ((int64_t)pair * max_splits + split) * g + col;
+#pragma unroll
+        for (int t = 0; t < HD / 16; ++t)
+          put<true>(reinterpret_cast<f32x4*>(ph.part_acc + slot * HD + 16 * t + 4 * g4), st.acc[0][t]);
+        if (g4 == 0) {
+          put<true>(ph.part_ml + slot * 2, st.m[0]);
+          put<true>(ph.part_ml + slot * 2 + 1, l);
+        }
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every lane's partial has arrived
+      int ticket = 0;
+      if (lane == 0)
+        ticket = __hip_atomic_fetch_add(ph.ticket_counters + pair, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      ticket = __builtin_amdgcn_readfirstlane(ticket);
+      asm volatile("" ::: "memory");
+      if (ticket == s_last - s_first) {
+        if (lane == 0) __hip_atomic_store(ph.ticket_counters + pair, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        to_merge = pair;
+      }
+    }
+    if (wq == 0 && lane == 0) s_flag[quad] = to_merge;
+    __syncthreads();
+    bool any = false;  // the same in the whole workgroup
+#pragma unroll
+    for (int qd = 0; qd < PROG_QUADS; ++qd) any = any || s_flag[qd] >= 0;
+    if (!any) continue;
+    const int pair = s_flag[quad];
+    // the merging quad: wavefront w adds the splits s_first + w, + 4, ... of every (head, four features)
+    // in split order (loads of eight splits in flight together) and leaves its sums in LDS
+    int m_first = 0, m_count = 0, m_tok = 0, m_kvh = 0;
+    if (pair >= 0) {
+      const int4 mw = ph.dec_work[pair / nkv];
+      m_tok = mw.x;
+      m_kvh = pair % nkv;
+      const int mstart = (window > 0 && mw.y - window + 1 > 0) ? mw.y - window + 1 : 0;
+      m_first = mstart / PROG_SPLIT;
+      m_count = mw.y / PROG_SPLIT - m_first + 1;
+      // the partials were written through by quads of any die while this die's L2 may still hold what
+      // an earlier step left at their addresses
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      for (int it = lane; it < merge_items; it += PAE_WAVE) {
+        const int c = it / (HD / 4), d = (it % (HD / 4)) * 4;
+        const int64_t slot0 = ((int64_t)pair * max_splits + m_first) * g + c;
+        float m = NEG_BIG, l = 0.f;
+        f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+        for (int sp = wq; sp < m_count; sp += 4) {
+          const int64_t slot = slot0 + (int64_t)sp * g;
+          const float ms = ph.part_ml[slot * 2], ls = ph.part_ml[slot * 2 + 1];
+          const f32x4 v = *reinterpret_cast<const f32x4*>(ph.part_acc + slot * HD + d);
+          const float m_new = fmaxf(m, ms);
+          const float f_old = exp2f(m - m_new), f = exp2f(ms - m_new);
+          a = a * f_old + v * f;
+          l = l * f_old + ls * f;
+          m = m_new;
+        }
+        float* dst = quad_lds + ((int64_t)wq * merge_items + it) * 6;
+        dst[0] = a[0]; dst[1] = a[1]; dst[2] = a[2]; dst[3] = a[3]; dst[4] = m; dst[5] = l;
+      }
+    }
+    __syncthreads();
+    if (pair >= 0) {
+      for (int it = wq * PAE_WAVE + lane; it < merge_items; it += 4 * PAE_WAVE) {
+        const int c = it / (HD / 4), d = (it % (HD / 4)) * 4;
+        const float* own = quad_lds + (int64_t)it * 6;
+        f32x4 a = {own[0], own[1], own[2], own[3]};
+        float m = own[4], l = own[5];
+        for (int other = 1; other < 4; ++other) {
+          const float* src = quad_lds + ((int64_t)other * merge_items + it) * 6;
+          const float ms = src[4], ls = src[5];
+          const float m_new = fmaxf(m, ms);
+          const float f_old = exp2f(m - m_new), f = exp2f(ms - m_new);
+          a = a * f_old + (f32x4){src[0], src[1], src[2], src[3]} * f;
+          l = l * f_old + ls * f;
+          m = m_new;
+        }
+        const float inv = 1.0f / l;
+        s16x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = bf16_bits(a[i] * inv);
+        put<true>(reinterpret_cast<s16x4*>(ph.attn_out + (int64_t)m_tok * ph.out_stride + (int64_t)(m_kvh * g + c) * HD + d), w);
+      }
+    }
+    __syncthreads();  // the quads' LDS is free for the next round
+  }
+}
+
+__global__ __launch_bounds__(PROG_THREADS) void decode_program_kernel(const ProgPhase* phases, int num_phases,
+                                                                      ProgBarrier* bar, int* host_error,
+                                                                      int quad_floats, int spin_limit) {
+  extern __shared__ float s_mem[];
+  __shared__ int s_flag[PROG_QUADS];
+  __shared__ int s_dead;
+  // The phase's description lives in LDS while the phase runs (read from memory, every use of a field
+  // after a store or a fence would be a trip of its own), and the next phase's is fetched before the
+  // barrier, so that its trip is over when the barrier opens.
+  __shared__ __align__(16) ProgPhase s_phase[3];
+  constexpr int PIECES = (int)(sizeof(ProgPhase) / 16);
+  int4 piece = {};  // this thread's 16 bytes of a coming phase's description, on their way
+  auto ask_for_phase = [&](int p) {
+    if (threadIdx.x < PIECES) piece = reinterpret_cast<const int4*>(phases + p)[threadIdx.x];
+  };
+  auto keep_phase = [&](int p) {
+    if (threadIdx.x < PIECES) reinterpret_cast<int4*>(&s_phase[p % 3])[threadIdx.x] = piece;
+  };
+  float* quad_lds = s_mem + (int64_t)(threadIdx.x / (4 * PAE_WAVE)) * quad_floats;
+  unsigned epoch = 0;
+  if (threadIdx.x == 0) {
+    s_dead = 0;
+    epoch = barrier_epoch_at_start(bar);
+  }
+  // phase p runs from s_phase[p % 3]; the description of phase p + 1 is there as well (a quad asks for
+  // its first weights of the next phase before the barrier), and that of phase p + 2 is on its way
+  ask_for_phase(0);
+  keep_phase(0);
+  if (num_phases > 1) {
+    ask_for_phase(1);
+    keep_phase(1);
+  }
+  __syncthreads();
+  int parity = 0;
+  Ahead ahead;
+  ahead.has_w = ahead.has_a = false;
+  for (int p = 0; p < num_phases; ++p) {
+    const ProgPhase& ph = s_phase[p % 3];
+    const ProgPhase* next = p + 1 < num_phases ? &s_phase[(p + 1) % 3] : nullptr;
+    if (p + 2 < num_phases) ask_for_phase(p + 2);  // kept when this phase is over
+    if (ph.type == PROG_PRODUCT) {
+      product_phase(ph, next, quad_lds, parity, ahead);
+    } else {
+      if (ph.hd == 128) attention_phase<128>(ph, quad_lds, s_flag);
+      else attention_phase<64>(ph, quad_lds, s_flag);
+      ahead = Ahead{};  // nothing is carried across an attention phase (and the registers are free during it)
+    }
+    if (p + 1 == num_phases) break;
+    // into the buffer of phase p - 1, whose last readers passed the barrier's workgroup barriers a phase ago
+    if (p + 2 < num_phases) keep_phase(p + 2);
+    if (!grid_barrier(bar, epoch, &s_dead, spin_limit, p)) {
+      if (threadIdx.x == 0 && blockIdx.x == 0) *host_error = p + 1;
+      return;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------- host side
+extern "C" int pae_program_phase_bytes() { return (int)sizeof(ProgPhase); }
+extern "C" int pae_program_barrier_bytes() { return (int)sizeof(ProgBarrier); }
+extern "C" int pae_program_max_rows() { return PROG_MAX_ROWS; }
+
+static int quad_bytes_of_product() { return 2 * 3 * 4 * PAE_WAVE * (int)sizeof(float); }
+
+// Writes phase `index` of the host-side list `phases`: a product with any epilogue but the rotating
+// one.  Arguments as pae_gemm_skinny; the k ranges are those that call would take.  Returns the
+// bytes of LDS a quad needs for the phase, or a negative code.
+extern "C" int pae_program_put_product(void* phases, int index, int epilogue, void* out, int64_t ldc, const void* A,
+                                       int64_t lda, const void* W, const void* bias, int b_is_f32, int M, int N, int K,
+                                       int splits, float* ticket_parts, int* ticket_counters, const float* row_stats,
+                                       int row_stat_tiles, float row_eps, void* next_rows, int64_t ld_next,
+                                       const void* next_w, int next_w_is_f32, float* next_stats, const SkinnyRope* rope) {
+  PAE_REQUIRE(phases && index >= 0, "decode program: no room for phase %d", index);
+  PAE_REQUIRE(M >= 1 && M <= PROG_MAX_ROWS, "decode program: a product of %d rows (1..%d are taken)", M, PROG_MAX_ROWS);
+  PAE_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && lda % 8 == 0, "decode program: N=%d K=%d lda=%lld (K and lda must be multiples of 8)",
+              N, K, (long long)lda);
+  PAE_REQUIRE(epilogue == EPI_BF16 || epilogue == EPI_F32 || epilogue == EPI_SWIGLU || epilogue == EPI_RESIDUAL ||
+              (epilogue == EPI_ROPE && rope), "decode program: unknown epilogue %d", epilogue);
+  const bool ticketed = splits > 1 && epilogue != EPI_F32;
+  PAE_REQUIRE(splits >= 1 && (!ticketed || (ticket_parts && ticket_counters)),
+              "decode program: %d k ranges with epilogue %d need scratch for partial sums and tickets", splits, epilogue);
+  PAE_REQUIRE(!(bias && splits > 1 && !ticketed), "decode program: a bias cannot be combined with partial sums");
+  PAE_REQUIRE(!row_stats || row_stat_tiles > 0, "decode program: a row scale needs its shares of the sums of squares");
+  PAE_REQUIRE(epilogue != EPI_RESIDUAL || (next_rows && next_w && next_stats && ld_next >= N && !bias),
+              "decode program: the residual epilogue needs the next rows, the next norm's weight and room for its sums, and takes no bias");
+  PAE_REQUIRE(epilogue != EPI_SWIGLU || (N % 16 == 0 && ldc % 4 == 0), "decode program: gated epilogue needs N %% 16 == 0, got %d", N);
+  PAE_REQUIRE(epilogue != EPI_ROPE || N % 16 == 0, "decode program: the rotating epilogue needs whole tiles, N=%d", N);
+  int k_per_split = (K + splits - 1) / splits;
+  k_per_split = (k_per_split + 127) / 128 * 128;
+  PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "decode program: %d k ranges are too many for K=%d", splits, K);
+  ProgPhase ph = {};
+  ph.type = PROG_PRODUCT;
+  ph.epilogue = epilogue;
+  ph.M = M; ph.N = N; ph.K = K; ph.splits = splits; ph.k_per_split = k_per_split; ph.b_is_f32 = b_is_f32;
+  ph.W = (const bf16_t*)W; ph.bias = bias; ph.A = (const bf16_t*)A; ph.out = out;
+  ph.lda = lda; ph.ldc = ldc;
+  ph.norm = SkinnyNorm{row_stats, row_stat_tiles, row_eps, (bf16_t*)next_rows, ld_next, next_w, next_w_is_f32, next_stats};
+  if (rope) ph.rope = *rope;
+  ph.ticket_parts = ticketed ? ticket_parts : nullptr;
+  ph.ticket_counters = ticketed ? ticket_counters : nullptr;
+  ((ProgPhase*)phases)[index] = ph;
+  return quad_bytes_of_product();
+}
+
+// The query/key/value product with rotation and cache write; arguments as pae_gemm_skinny_rope.
+extern "C" int pae_program_put_product_rope(void* phases, int index, void* q_out, int64_t ldq, const void* A, int64_t lda,
+                                            const void* W, const void* bias, int b_is_f32, int M, int K, int nh, int nkv,
+                                            int hd, int rot, const float* cos_sin, const int* positions,
+                                            const int* tok_seq, const int* block_tables, int max_blocks, int bs,
+                                            void* k_cache, void* v_cache, int splits, float* ticket_parts,
+                                            int* ticket_counters, const float* row_stats, int row_stat_tiles,
+                                            float row_eps) {
+  PAE_REQUIRE(nh > 0 && nkv >= 0 && hd > 0 && hd % 16 == 0, "decode program: bad head sizes nh=%d nkv=%d hd=%d", nh, nkv, hd);
+  PAE_REQUIRE(rot >= 0 && rot <= hd && rot % 16 == 0 && (rot == 0 || cos_sin),
+              "decode program: rotary_dim %d must be a multiple of 16 up to head_dim %d", rot, hd);
+  PAE_REQUIRE(ldq >= (int64_t)nh * hd && ldq % 4 == 0, "decode program: row stride %lld of the queries", (long long)ldq);
+  PAE_REQUIRE(positions, "decode program: positions are missing");
+  PAE_REQUIRE(nkv == 0 || (bs > 0 && max_blocks > 0 && k_cache && v_cache && block_tables && tok_seq),
+              "decode program: the cache write needs tables and pools");
+  const SkinnyRope rope{cos_sin, positions, tok_seq, block_tables, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                        nh, nkv, hd, rot, max_blocks, bs};
+  return pae_program_put_product(phases, index, EPI_ROPE, q_out, ldq, A, lda, W, bias, b_is_f32, M, (nh + 2 * nkv) * hd, K,
+                                 splits, ticket_parts, ticket_counters, row_stats, row_stat_tiles, row_eps, nullptr, 0,
+                                 nullptr, 0, nullptr, &rope);
+}
+
+// Decode attention of num_dec tokens; arguments as pae_attn_decode_bf16, plus one ticket counter
+// (zero before and after) per (token, key/value head).
+extern "C" int pae_program_put_attention(void* phases, int index, void* out, int64_t out_stride, const void* q,
+                                         int64_t q_stride, const void* k_cache, const void* v_cache, const int* dec_work,
+                                         int num_dec, const int* block_tables, int max_blocks, int bs, int nh, int nkv,
+                                         int hd, float scale, int window, void* part_acc, void* part_ml,
+                                         int* ticket_counters) {
+  PAE_REQUIRE(phases && index >= 0, "decode program: no room for phase %d", index);
+  PAE_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0 && nh / nkv <= 16, "decode program: %d query heads over %d key/value heads", nh, nkv);
+  PAE_REQUIRE(hd == 64 || hd == 128, "decode program: attention takes head_dim 64 or 128, got %d", hd);
+  PAE_REQUIRE(nh / nkv * (hd / 4) <= PROG_MERGE_ITEMS, "decode program: %d heads of %d features per key/value head exceed the merge",
+              nh / nkv, hd);
+  PAE_REQUIRE(bs >= 16 && bs % 16 == 0 && max_blocks > 0 && window >= 0, "decode program: page size %d, table width %d, window %d",
+              bs, max_blocks, window);
+  PAE_REQUIRE(num_dec >= 1 && num_dec <= PROG_MAX_ROWS && dec_work && block_tables && part_acc && part_ml && ticket_counters,
+              "decode program: attention of %d tokens (1..%d are taken) needs its work list, tables, scratch and tickets",
+              num_dec, PROG_MAX_ROWS);
+  ProgPhase ph = {};
+  ph.type = PROG_ATTENTION;
+  ph.dec_work = (const int4*)dec_work; ph.block_tables = block_tables;
+  ph.q = (const bf16_t*)q; ph.attn_out = (bf16_t*)out;
+  ph.k_cache = (const bf16_t*)k_cache; ph.v_cache = (const bf16_t*)v_cache;
+  ph.part_acc = (float*)part_acc; ph.part_ml = (float*)part_ml;
+  ph.q_stride = q_stride; ph.out_stride = out_stride;
+  ph.num_dec = num_dec;
+  ph.max_splits = (int)(((int64_t)max_blocks * bs + PROG_SPLIT - 1) / PROG_SPLIT);
+  ph.max_blocks = max_blocks; ph.bs = bs; ph.nh = nh; ph.nkv = nkv; ph.hd = hd; ph.window = window;
+  ph.scale_log2 = scale * LOG2E;
+  ph.ticket_counters = ticket_counters;
+  ((ProgPhase*)phases)[index] = ph;
+  const int state = 3 * (hd / 4 + 2) * PAE_WAVE, merge = 4 * (nh / nkv) * (hd / 4) * 6;
+  return (state > merge ? state : merge) * (int)sizeof(float);
+}
+
+// The most workgroups that can be resident at once on the current device (one per compute unit at the
+// kernel's 1,024 threads); also asks the runtime for the kernel's LDS.  Call it once per device before
+// the first pae_program_run there, outside any stream capture.
+#define PROG_LDS_LIMIT (160 * 1024 - 2048)  // dynamic LDS: what the kernel declares for itself (phase descriptions, flags) stays below 2 KB
+static int g_max_groups[64];
+
+extern "C" int pae_program_max_groups() {
+  int dev = 0, units = 0, per_unit = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess || dev < 0 || dev >= 64) return pae_fail("decode program: no usable current device");
+  if (g_max_groups[dev] > 0) return g_max_groups[dev];
+  err = hipFuncSetAttribute((const void*)decode_program_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, PROG_LDS_LIMIT);
+  if (err != hipSuccess) return pae_fail("decode program: cannot ask for LDS: %s", hipGetErrorString(err));
+  err = hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev);
+  if (err == hipSuccess)
+    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_unit, (const void*)decode_program_kernel, PROG_THREADS,
+                                                       PROG_LDS_LIMIT);
+  if (err != hipSuccess) return pae_fail("decode program: cannot tell how many workgroups fit: %s", hipGetErrorString(err));
+  PAE_REQUIRE(units * per_unit >= 1, "decode program: the kernel does not fit a compute unit");
+  g_max_groups[dev] = units * per_unit;
+  return g_max_groups[dev];
+}
+
+// Runs phases[0 .. num_phases) (device memory) on `groups` resident workgroups.  `barrier` is
+// pae_program_barrier_bytes() of device memory, zero before its first use and used with one value of
+// `groups` only; `host_error` is an int in pinned host memory that receives 1 + the phase at whose
+// barrier a workgroup gave up after `spin_limit` polls (it stays as it is otherwise).  Launches that
+// share a barrier block or ticket counters must not overlap.
+extern "C" int pae_program_run(const void* phases, int num_phases, void* barrier, int* host_error, int groups,
+                               int quad_lds_bytes, int spin_limit, hipStream_t stream) {
+  PAE_REQUIRE(phases && barrier && host_error && num_phases >= 1, "decode program: nothing to run");
+  PAE_REQUIRE(quad_lds_bytes >= quad_bytes_of_product() && quad_lds_bytes % 16 == 0 && quad_lds_bytes * PROG_QUADS <= PROG_LDS_LIMIT,
+              "decode program: %d bytes of LDS a quad", quad_lds_bytes);
+  PAE_REQUIRE(spin_limit > 0, "decode program: the waits must be bounded");
+  int dev = 0;
+  PAE_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && g_max_groups[dev] > 0,
+              "decode program: pae_program_max_groups has not been called on this device");
+  // every workgroup must be resident at once, or the barrier between the phases never completes
+  PAE_REQUIRE(groups >= 1 && groups <= g_max_groups[dev], "decode program: %d workgroups cannot all be resident (at most %d)",
+              groups, g_max_groups[dev]);
+  decode_program_kernel<<<groups, PROG_THREADS, (size_t)quad_lds_bytes * PROG_QUADS, stream>>>(
+      (const ProgPhase*)phases, num_phases, (ProgBarrier*)barrier, host_error, quad_lds_bytes / (int)sizeof(float), spin_limit);
+  return pae_check_launch("decode program");
+}

@@ -20,321 +20,7 @@
 // makes a round trip through memory.
 #include "common.h"
 #include "api.h"
-
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-
-#define EPI_BF16 0
-#define EPI_F32 1
-#define EPI_SWIGLU 2
-#define EPI_ROPE 3
-#define EPI_RESIDUAL 4
-
-// RMS normalisation folded into the products around it, so that a decode step needs no norm
-// kernel between them.  norm(x) W^T = rsqrt(mean(x^2) + eps) * ((x * w_norm) W^T): the scale is one
-// number per row and can be applied to the finished sums.
-//
-// Producer (EPI_RESIDUAL, the product that ends a residual branch): the sums of all k ranges are
-// added into the float32 residual in place; the same tile is written again as
-// bfloat16(residual * w_next), the rows the next product multiplies, and the tile's share of every
-// row's sum of squares goes to next_stats[m][16-column tile].
-// Consumer (any epilogue): `row_stats` holds those shares for the rows of A; every lane adds up
-// its row's shares in a fixed order (the same in every workgroup, so all columns of a row get the
-// same scale) and multiplies its sums by rsqrt(total / K + eps) before bias, rotation or gate.
-struct SkinnyNorm {
-  const float* row_stats;  // [M][row_stat_tiles] or null: A's rows are used as they are
-  int row_stat_tiles;
-  float eps;
-  bf16_t* next_rows;       // EPI_RESIDUAL: [M][ld_next] bfloat16(residual * next_w)
-  int64_t ld_next;
-  const void* next_w;      // [N] weight of the norm that follows
-  int next_w_is_f32;
-  float* next_stats;       // [M][(N + 15) / 16]
-};
-
-// rsqrt(mean of squares + eps) of row m of A from the shares the producer left.  The four lanes
-// that hold row m (g4 = 0..3) read the shares 16 bytes at a time, all reads of a batch of up to
-// 128 shares in flight at once (a loop that adds one share after the other waits out the memory's
-// latency once per share), add theirs in index order and then each other's: the same order in every
-// workgroup, so every column of a row is scaled by the same number.
-__device__ __forceinline__ float row_scale_of(const SkinnyNorm& norm, int m, int g4, float inv_width) {
-  const float* shares = norm.row_stats + (int64_t)m * norm.row_stat_tiles;
-  const int tiles = norm.row_stat_tiles;
-  const bool aligned = tiles % 4 == 0;  // rows of shares then start on 16-byte boundaries
-  float sum = 0.f;
-  for (int base = 0; base < tiles; base += 128) {
-    f32x4 part[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int t = base + 16 * u + 4 * g4;
-      if (aligned && t + 4 <= tiles) {
-        part[u] = *reinterpret_cast<const f32x4*>(shares + t);
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) part[u][i] = t + i < tiles ? shares[t + i] : 0.f;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) sum += (part[u][0] + part[u][1]) + (part[u][2] + part[u][3]);
-  }
-  sum += __shfl_xor(sum, 16);
-  sum += __shfl_xor(sum, 32);
-  return rsqrtf(sum * inv_width + norm.eps);
-}
-
-// The scales of this lane's rows of A (row 16 mt + lane % 16 of column tile mt), 1 without a folded
-// norm.  Asked for at the start of a kernel, so that the shares arrive while the products run.
-template <int MT>
-__device__ __forceinline__ void row_scales(float (&scale)[MT], const SkinnyNorm& norm, int M, int K) {
-  const int lane = threadIdx.x % PAE_WAVE;
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = 16 * mt + lane % 16;
-    scale[mt] = norm.row_stats ? row_scale_of(norm, m < M ? m : M - 1, lane / 16, 1.0f / (float)K) : 1.0f;
-  }
-}
-
-// What the rotating epilogue needs beside the product: the head geometry, the
-// rotation's frequencies, every row's position and sequence, and the paged cache.
-struct SkinnyRope {
-  const float* cos_sin;     // [M][rot / 2][2] cosine and sine of every row's angles, or null without rotation
-  const int* positions;     // [M]
-  const int* tok_seq;       // [M] row of block_tables
-  const int* block_tables;  // [sequences][max_blocks]
-  bf16_t* k_cache;          // [block][kv head][bs][hd]
-  bf16_t* v_cache;          // [block][kv head][hd][bs]
-  int nh, nkv, hd, rot, max_blocks, bs;
-};
-
-// Feature within its head of row `r` of the `j`-th tile of a head: a tile inside the rotated
-// part holds features 8 j .. 8 j + 7 (rows 0-7) and their partners rot / 2 + 8 j .. (rows 8-15);
-// tiles past it hold 16 consecutive features that pass through.
-__device__ __forceinline__ int rope_feature(int j, int r, int rot) {
-  return 16 * j < rot ? (r < 8 ? 8 * j + r : rot / 2 + 8 * j + r - 8) : 16 * j + r;
-}
-
-// A fragment loaded as (row = lane / 4, k group = lane % 4) moved to (row = lane % 16, k group = lane / 16).
-__device__ __forceinline__ bf16x8 to_mfma_order(bf16x8 v, int fetch_from) {
-  typedef __attribute__((ext_vector_type(4))) int i32x4;
-  i32x4 raw = *reinterpret_cast<i32x4*>(&v);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) raw[i] = __builtin_amdgcn_ds_bpermute(fetch_from, raw[i]);
-  return *reinterpret_cast<bf16x8*>(&raw);
-}
-
-__device__ __forceinline__ short to_bf16_bits(float x) {
-  const bf16_t h = __float2bfloat16(x);
-  return *reinterpret_cast<const short*>(&h);
-}
-
-// What a wavefront does with finished sums: acc[rt][mt] is the 16 x 16 tile of weight rows
-// 16 (tile_base + rt) .. (through the rotation's row order, if any) by rows 16 mt .. of A; a lane
-// holds row m = 16 mt + lane % 16 of A and weight rows 4 (lane / 16) + i.  only_mt >= 0: just
-// that column tile (the others belong to other wavefronts).
-template <int MT, int RT, int EPI>
-__device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int tile_base, int only_mt,
-                                                void* __restrict__ out, int64_t ldc, const void* __restrict__ bias,
-                                                int b_is_f32, int M, int N, int split, int64_t part_stride,
-                                                const SkinnyRope& rope, const SkinnyNorm& norm,
-                                                const float (&scale)[MT]) {
-  const int lane = threadIdx.x % PAE_WAVE;
-  const int r = lane % 16, g4 = lane / 16;
-  if (EPI == EPI_ROPE) {
-    // lane holds row m = 16 mt + r of A and rows 4 g4 + i of each tile: lanes 0-31 the lower
-    // features of the pairs, lanes 32-63 (same m) their partners
-    const int per_head = rope.hd / 16;
-    const int64_t head_step = (int64_t)rope.bs * rope.hd;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      if (only_mt >= 0 && mt != only_mt) continue;  // another wavefront's column tile
-      const int m = 16 * mt + r;
-      const int mc = m < M ? m : M - 1;
-      const int pos = rope.positions[mc];
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int tile = tile_base + rt;
-        const int head = tile / per_head, j = tile % per_head;
-        const bool rotated = 16 * j < rope.rot && head < rope.nh + rope.nkv;  // values keep the tile layout, unrotated
-        const int f0 = rope_feature(j, 4 * g4, rope.rot);  // first of this lane's 4 consecutive features
-        const int n = head * rope.hd + f0;
-        s16x4 res;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          // the projection is rounded to bfloat16 before the rotation, as where the two are separate kernels
-          const float own = __bfloat162float(__float2bfloat16(
-              acc[rt][mt][i] * scale[mt] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f)));
-          const float other = __shfl_xor(own, 32);  // in every lane
-          float o = own;
-          if (rotated) {
-            const float* angle = rope.cos_sin + ((int64_t)mc * (rope.rot / 2) + 8 * j + (4 * g4 + i) % 8) * 2;
-            const float cs = angle[0], sn = angle[1];
-            o = g4 < 2 ? own * cs - other * sn : own * cs + other * sn;
-          }
-          res[i] = to_bf16_bits(o);
-        }
-        if (m >= M || n >= N) continue;
-        if (head < rope.nh) {
-          *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + n) = res;
-          continue;
-        }
-        const int off = pos % rope.bs;
-        const int64_t page = (int64_t)rope.block_tables[(int64_t)rope.tok_seq[m] * rope.max_blocks + pos / rope.bs] *
-                             rope.nkv * head_step;
-        if (head < rope.nh + rope.nkv) {
-          *reinterpret_cast<s16x4*>(rope.k_cache + page + (head - rope.nh) * head_step + (int64_t)off * rope.hd + f0) = res;
-        } else {
-          short* dst = reinterpret_cast<short*>(rope.v_cache) + page + (head - rope.nh - rope.nkv) * head_step +
-                       (int64_t)f0 * rope.bs + off;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) dst[(int64_t)i * rope.bs] = res[i];
-        }
-      }
-    }
-    return;
-  }
-
-  const bool vec = ldc % 4 == 0;  // rows of out keep 8- and 16-byte stores aligned
-  // lane holds, per column tile mt, row m = 16 mt + r of A and weight rows 4 g4 + i of each row tile
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    if (only_mt >= 0 && mt != only_mt) continue;  // another wavefront's column tile
-    const int m = 16 * mt + r;
-    if (m >= M) continue;
-    if (EPI == EPI_SWIGLU) {
-      // a tile holds 8 gate rows (lanes 0-31: rows 4 g4 + i) and their 8 up rows (lanes 32-63, same m)
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int j = (tile_base + rt) * 8 + 4 * (g4 % 2);  // output feature of register 0
-        s16x4 v;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float own = acc[rt][mt][i] * scale[mt];
-          const float up = __shfl_xor(own, 32);  // in every lane (the same row of A, so the same scale)
-          v[i] = to_bf16_bits(own / (1.0f + expf(-own)) * up);
-        }
-        if (g4 < 2 && j < N / 2)  // N counts gate and up rows
-          *reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j) = v;
-      }
-    } else if (EPI == EPI_RESIDUAL) {
-      // residual += sums; the next product's rows and this tile's share of the row's sum of squares
-      float* res = (float*)out + (int64_t)m * ldc;
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int n = 16 * (tile_base + rt) + 4 * g4;
-        float ss = 0.f;
-        if (n < N) {
-          float v[4];
-          s16x4 p;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const bool in = n + i < N;
-            v[i] = in ? res[n + i] + acc[rt][mt][i] * scale[mt] : 0.f;
-            ss += v[i] * v[i];
-            p[i] = to_bf16_bits(in ? v[i] * load_param(norm.next_w, norm.next_w_is_f32, n + i) : 0.f);
-          }
-          bf16_t* nxt = norm.next_rows + (int64_t)m * norm.ld_next + n;
-          if (vec && norm.ld_next % 4 == 0 && n + 4 <= N) {
-            *reinterpret_cast<f32x4*>(res + n) = (f32x4){v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<s16x4*>(nxt) = p;
-          } else {
-            for (int i = 0; i < 4 && n + i < N; ++i) {
-              res[n + i] = v[i];
-              reinterpret_cast<short*>(nxt)[i] = p[i];
-            }
-          }
-        }
-        ss += __shfl_xor(ss, 16);  // the four lanes that hold this row's 16 columns
-        ss += __shfl_xor(ss, 32);
-        if (g4 == 0 && 16 * (tile_base + rt) < N) norm.next_stats[(int64_t)m * ((N + 15) / 16) + tile_base + rt] = ss;
-      }
-    } else {
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int n = 16 * (tile_base + rt) + 4 * g4;
-        if (n >= N) continue;
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          v[i] = acc[rt][mt][i] * scale[mt] + ((bias && n + i < N) ? load_param(bias, b_is_f32, n + i) : 0.f);
-        if (EPI == EPI_F32) {
-          float* dst = (float*)out + (int64_t)split * part_stride + (int64_t)m * ldc + n;
-          if (vec && n + 4 <= N) *reinterpret_cast<f32x4*>(dst) = (f32x4){v[0], v[1], v[2], v[3]};
-          else
-            for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = v[i];
-        } else {
-          bf16_t* dst = (bf16_t*)out + (int64_t)m * ldc + n;
-          if (vec && n + 4 <= N) {
-            s16x4 p;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) p[i] = to_bf16_bits(v[i]);
-            *reinterpret_cast<s16x4*>(dst) = p;
-          } else
-            for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = __float2bfloat16(v[i]);
-        }
-      }
-    }
-  }
-}
-
-// Several k ranges for an epilogue that needs whole sums (bias, rotation, gate): every range's
-// workgroup leaves its partial tile in `parts` and draws a ticket from the tile's counter; the one
-// that draws the last ticket knows that all partials are written, adds them in range order
-// whichever workgroup it is (so the sums do not depend on the order of arrival), puts the counter
-// back to zero and runs the epilogue.  Nobody waits for anybody.
-//
-// Why relaxed device-scope atomics and one wait are enough here (gfx942/gfx950).  The chip is eight
-// dies, each with an L2 of its own that is not kept coherent with the others'; the memory side behind
-// them (the shared last-level cache and HBM) is the point at which all dies agree.  A device-scope
-// ("agent") atomic store or load is issued with the sc1 bit: the store is written through to that
-// point and the load is served from it, whatever either die's L2 holds.  `s_waitcnt vmcnt(0)` returns
-// when every vector memory operation of the wavefront, these stores included, has been
-// acknowledged, which for a written-through store means that it has arrived there.  So: (1) a
-// workgroup's partial sums are at the common point before it draws its ticket; (2) the ticket is a
-// device-scope read-modify-write, carried out at the same point, so tickets are handed out in one
-// order, and whoever draws the last one does so after every other range's partials have arrived;
-// (3) its loads of the partials are issued after the ticket's value has come back (they sit behind a
-// branch on that value and a compiler barrier) and, being sc1 loads, cannot be served stale from a
-// cache.  A release fence would add a write-back of the die's whole L2 (`buffer_wbl2`) for the sake
-// of ordinary stores that may still be dirty there; there are none that matter, because the
-// partials never were ordinary stores (measured: 13 us a launch with the fence, 1 us without).
-// The counters are shared by every launch on a device: the launches must not overlap, which the
-// host side enforces by tying the counters to one stream.
-struct SkinnyTickets {
-  float* parts;   // [slots][k ranges][RT * 4][64]: a wavefront's accumulators, lane by lane
-  int* counters;  // [slots], zero before and after every launch; null: one k range
-};
-
-// True in the wavefront that holds the whole sums afterwards (in `acc`); the others are done.
-template <int RT>
-__device__ __forceinline__ bool add_up_k_ranges(f32x4 (&acc)[RT], int slot, int split, int splits,
-                                                const SkinnyTickets& tk) {
-  const int lane = threadIdx.x % PAE_WAVE;
-  float* mine = tk.parts + ((int64_t)slot * splits + split) * (RT * 4 * PAE_WAVE) + lane;
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __hip_atomic_store(mine + (rt * 4 + i) * PAE_WAVE, acc[rt][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every lane's stores have arrived
-  int ticket = 0;
-  if (lane == 0) ticket = __hip_atomic_fetch_add(tk.counters + slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  ticket = __builtin_amdgcn_readfirstlane(ticket);
-  asm volatile("" ::: "memory");
-  if (ticket != splits - 1) return false;  // the same in every lane
-  if (lane == 0) __hip_atomic_store(tk.counters + slot, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) acc[rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int p = 0; p < splits; ++p) {
-    const float* theirs = tk.parts + ((int64_t)slot * splits + p) * (RT * 4 * PAE_WAVE) + lane;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        acc[rt][i] += __hip_atomic_load(theirs + (rt * 4 + i) * PAE_WAVE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  return true;
-}
+#include "skinny_device.h"
 
 // MT: column tiles of 16 rows of A; RT: tiles of 16 weight rows per workgroup; SKINNY_U: k steps
 // of a wavefront whose loads are in flight together.  With more
@@ -347,7 +33,11 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
                                                           const void* __restrict__ bias, int b_is_f32, int M,
                                                           int N, int K, int k_per_split, int64_t part_stride,
                                                           SkinnyRope rope, SkinnyTickets tickets, SkinnyNorm norm) {
-  static_assert(NW == 4 || MT == 1, "more than four wavefronts only with one column tile");
+  // NW == 16 (one column tile only): the workgroup holds four k ranges side by side, four wavefronts to
+  // each, and adds the ranges' sums in range order itself: the sums, bit for bit, of four workgroups
+  // with one range each whose results the last to finish adds up (grid.y == 4), without the tickets
+  // and the trip to memory.
+  static_assert(NW == 4 || (NW == 16 && MT == 1), "sixteen wavefronts only with one column tile");
   __shared__ float s_part[MT == 1 ? NW - 1 : 4][RT * MT * 4][PAE_WAVE];
   if (MT == 1 && gridDim.z > 1) {  // the rows of A are shared out in tiles of 16: this workgroup's tile
     const int m0 = blockIdx.z * 16;
@@ -370,7 +60,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
   const int r = lane % 16, g4 = lane / 16;
   float scale[MT];
   const int n0 = blockIdx.x * 16 * RT;
-  const int k_lo = blockIdx.y * k_per_split;
+  const int k_lo = (NW == 16 ? wave / 4 : blockIdx.y) * k_per_split;
   const int k_hi = min(K, k_lo + k_per_split);
 
   // Loads are made with the lane order (row = lane / 4, k group = lane % 4): the four lanes of a
@@ -406,7 +96,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
   // addresses, and issued SKINNY_U steps ahead of their use; a lane past the end of
   // the k range zeroes its weight fragment (rows past N or M are simply not stored).
   const bf16x8 zero = {};
-  constexpr int KW = 32 * NW;  // the workgroup's wavefronts take 32-wide k steps in turn
+  constexpr int KW = 128;  // a range's four wavefronts take 32-wide k steps in turn
   struct Batch {  // SKINNY_U steps of a wavefront: k offsets kb + KW u
     bf16x8 wf[SKINNY_U][RT], af[SKINNY_U][MT];
   };
@@ -441,7 +131,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
   };
   constexpr int STEP = KW * SKINNY_U;
   constexpr bool PIPELINED = true;
-  int kb = k_lo + 32 * wave;  // the same in every lane of a wavefront: the branches on it are uniform
+  int kb = k_lo + 32 * (wave % 4);  // the same in every lane of a wavefront: the branches on it are uniform
   if (PIPELINED) {
     // two batches take turns, so that a wavefront always has loads in flight: with one, every
     // batch waits out the memory's latency before the next is even asked for
@@ -479,11 +169,24 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
     __syncthreads();
     if (wave > 0) return;
 #pragma unroll
-    for (int w = 0; w < NW - 1; ++w)
+    for (int w = 0; w < 3; ++w)
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[rt][0][i] += s_part[w][rt * 4 + i][lane];
+    if (NW == 16) {  // the other three ranges: each added up in wavefront order, then onto the first in range order
+#pragma unroll
+      for (int range = 1; range < 4; ++range)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float sum = s_part[4 * range - 1][rt * 4 + i][lane];
+#pragma unroll
+            for (int w = 0; w < 3; ++w) sum += s_part[4 * range + w][rt * 4 + i][lane];
+            acc[rt][0][i] += sum;
+          }
+    }
   } else {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
@@ -681,8 +384,7 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + 127) / 128 * 128;
   PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "gemm_skinny: %d k ranges are too many for K=%d", splits, K);
-  // many weight rows and more than 8 rows of A: 128 weight rows a workgroup, activations through LDS
-  // (from 9 rows on: 7B gate/up at 16 rows 62.3 -> 55.3 us, 72B 230 -> 200 us)
+  // many weight rows and more than 16 rows of A: 128 weight rows a workgroup, activations through LDS
   // (measured at 1.5B/7B/72B layer sizes: ahead from about one workgroup per compute unit on, behind below)
   const int medium_groups = (N + 127) / 128;
   // Up to 48 rows of A and fewer than four such workgroups per compute unit: 64 weight rows a workgroup
@@ -693,7 +395,9 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   const bool only_narrow_fills = (int64_t)medium_groups * splits < 256 && (int64_t)narrow_groups * splits >= 384;
   const bool wide = !only_narrow_fills &&
                     (mt > 3 || (int64_t)medium_groups * splits >= 1024 || (int64_t)narrow_groups * splits < 512);
-  if (M > 8 && ((int64_t)medium_groups * splits >= 256 || only_narrow_fills)) {
+  // (up to 16 rows every product takes the first kernel, whose order of adding the decode program shares:
+  // a row's sums are then the same bits alone, in a batch, in a program or launched by itself)
+  if (M > 16 && ((int64_t)medium_groups * splits >= 256 || only_narrow_fills)) {
     dim3 mgrid(wide ? medium_groups : (N + 63) / 64, splits);
 #define LAUNCH_MEDIUM(MT, EPI)                                                                                   \
   if (wide)                                                                                                      \
@@ -740,14 +444,14 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
 #undef LAUNCH_TILED
     return pae_check_launch("gemm_skinny (rows of A in tiles)");
   }
-  if (epilogue == EPI_RESIDUAL && mt == 1 && splits == 1 && K >= 1024) {
-    // One k range, so that the sums are whole without tickets, and sixteen wavefronts to share it out:
-    // few workgroups, but each keeps its compute unit's memory pipeline full.  (The callers choose one
-    // range where that is ahead, see kernels/lib.py `residual_splits`; for the rotating epilogue sixteen
-    // wavefronts were slower at every size tried.)
+  if (epilogue == EPI_RESIDUAL && mt == 1 && splits == 4 && K >= 1024 && ((N + 15) / 16 >= 192 || 32 * (int64_t)K <= 65536)) {
+    // Four k ranges side by side in one workgroup of sixteen wavefronts: no tickets, no trip to memory
+    // for partial sums; few workgroups, but each keeps its compute unit's memory pipeline full.  Ahead
+    // wherever the 16-row workgroups fill the chip or have little to read each (1.5B O at 8 rows 7.2 ->
+    // 5.9 us, 7B down 38.3 -> 36.1 us); the same bits as the ticketed ranges (see the kernel).
     gemm_skinny_kernel<1, 1, EPI_RESIDUAL, 4, 16><<<dim3((N + 15) / 16, 1), 1024, 0, stream>>>(
         out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, bias, b_is_f32, M, N, K, k_per_split, part_stride, rope,
-        tickets, norm);
+        SkinnyTickets{nullptr, nullptr}, norm);
     return pae_check_launch("gemm_skinny (sixteen wavefronts)");
   }
   dim3 grid((N + 16 * rt - 1) / (16 * rt), splits);

@@ -232,22 +232,55 @@ static __device__ __align__(256) unsigned char scratch[PAE_SAMPLE_STATIC_BYTES];
 static void* g_scratch_of_device[PAE_MAX_DEVICES];
 static std::mutex g_scratch_mutex;
 
-static int scratch_on_current_device(void** out) {
-  int dev = -1;
-  hipError_t err = hipGetDevice(&dev);
+// The device a call works on is the one its stream belongs to (the null stream: the current device),
+// not whichever device happens to be current: kernels launched on that stream run there, and each GPU
+// has the buffer at an address of its own.
+static int device_of_stream(hipStream_t stream, int* out) {
+  int current = -1;
+  hipError_t err = hipGetDevice(&current);
   if (err != hipSuccess) return pae_fail("sample_static: no current device: %s", hipGetErrorString(err));
-  PAE_REQUIRE(dev >= 0 && dev < PAE_MAX_DEVICES, "sample_static: device %d beyond the %d this library keeps track of",
-              dev, PAE_MAX_DEVICES);
+  *out = current;
+  if (stream) {
+    hipDevice_t dev = -1;
+    err = hipStreamGetDevice(stream, &dev);
+    if (err != hipSuccess) return pae_fail("sample_static: cannot tell the stream's device: %s", hipGetErrorString(err));
+    *out = (int)dev;
+  }
+  PAE_REQUIRE(*out >= 0 && *out < PAE_MAX_DEVICES, "sample_static: device %d beyond the %d this library keeps track of",
+              *out, PAE_MAX_DEVICES);
+  return 0;
+}
+
+// The buffer's address on device `dev`, looked up at the first call for that device with that device
+// current (and the caller's device current again afterwards).  The lookup asks the runtime (it may load
+// the code object there), so it must not fall inside a stream capture: `capturing` refuses it then.
+static int scratch_on_device(int dev, bool capturing, void** out) {
   std::lock_guard<std::mutex> hold(g_scratch_mutex);
   if (!g_scratch_of_device[dev]) {
+    PAE_REQUIRE(!capturing, "sample_static: the first call on device %d falls inside a stream capture; call "
+                "pae_sample_static_prepare (or pae_sample_static once) on this device before capturing", dev);
+    int current = -1;
+    hipError_t err = hipGetDevice(&current);
+    if (err == hipSuccess && current != dev) err = hipSetDevice(dev);
+    if (err != hipSuccess) return pae_fail("sample_static: cannot make device %d current: %s", dev, hipGetErrorString(err));
     void* ptr = nullptr;
     err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (current != dev) (void)hipSetDevice(current);
     if (err != hipSuccess || !ptr)
       return pae_fail("sample_static: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(err));
     g_scratch_of_device[dev] = ptr;
   }
   *out = g_scratch_of_device[dev];
   return 0;
+}
+
+// Looks the buffer's address up for the current device, so that a later pae_sample_static there may
+// be issued inside a stream capture.  Allocates nothing.
+extern "C" int pae_sample_static_prepare() {
+  int dev = -1;
+  if (int code = device_of_stream(nullptr, &dev)) return code;
+  void* base = nullptr;
+  return scratch_on_device(dev, false, &base);
 }
 
 extern "C" int pae_sample_static_slots() { return PAE_SAMPLE_STATIC_SLOTS; }
@@ -260,8 +293,12 @@ extern "C" int pae_sample_static(int* tokens, const float* logits, int64_t ld, c
               "sample_static: %d rows of %d logits need %lld chunk slots, the built-in buffer holds %d "
               "(use pae_sample with a workspace of the caller's)",
               num_rows, vocab, (long long)slots, PAE_SAMPLE_STATIC_SLOTS);
+  int dev = -1;
+  if (int code = device_of_stream(stream, &dev)) return code;
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (stream && hipStreamIsCapturing(stream, &capture) != hipSuccess) capture = hipStreamCaptureStatusNone;
   void* base = nullptr;
-  if (int code = scratch_on_current_device(&base)) return code;
+  if (int code = scratch_on_device(dev, capture != hipStreamCaptureStatusNone, &base)) return code;
   double* chunk_sum = (double*)base;
   float* chunk_max = (float*)(chunk_sum + PAE_SAMPLE_STATIC_SLOTS);
   int* chunk_arg = (int*)(chunk_max + PAE_SAMPLE_STATIC_SLOTS);

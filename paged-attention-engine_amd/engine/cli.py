@@ -29,7 +29,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     p.add_argument("--seed", type=int, default=0, help="seed of the random weights")
     p.add_argument("--save-model", help="with --random-config: draw the weights on the CPU, write the model folder "
                    "here and load it")
-    p.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
+    p.add_argument("--dtype", choices=("bfloat16", "float32"), default=None,
+                   help="default: the torch_dtype of the model's config.json (bfloat16 if it is neither of the two)")
     p.add_argument("--prompt-ids", action="append", default=[], help='one prompt as "1,2,3" (repeatable)')
     p.add_argument("--prompts-file", help="one prompt of token ids per line")
     p.add_argument("--max-new-tokens", type=int, default=16)

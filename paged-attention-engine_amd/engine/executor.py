@@ -17,13 +17,17 @@ from .step import StepEntry, StepRunner
 class LaunchedStep:
     """A step that has been handed to the GPU: its tokens, and which row is whose."""
 
-    def __init__(self, tokens: SampledTokens, row_of: Dict[int, int], sampling: List) -> None:
+    def __init__(self, tokens: SampledTokens, row_of: Dict[int, int], sampling: List, runner=None) -> None:
         self.tokens = tokens
         self.row_of = row_of      # id(sequence) -> row of its token
         self.sampling = sampling  # the work items that sample, in row order
+        self.runner = runner
 
     def wait(self) -> List[int]:
-        return self.tokens.wait()
+        tokens = self.tokens.wait()
+        if self.runner is not None:
+            self.runner.check_programs()  # the step has finished: did its resident kernel get through?
+        return tokens
 
 
 class ModelExecutor:
@@ -47,6 +51,7 @@ class ModelExecutor:
         temperatures = [w.seq.request.temperature for w in sampling]
         uniforms = self._uniforms(sampling)
         tokens = self.sampler.sample(logits, temperatures, uniforms)
+        self.runner.check_programs()  # the tokens are on the host, so the step has finished
         rows = logits.cpu() if record_logits else None
         out, k = [], 0
         for w in work:
@@ -77,4 +82,4 @@ class ModelExecutor:
         temperatures = [w.seq.request.temperature for w in sampling]
         uniforms = self._uniforms(sampling)
         tokens = self.sampler.sample_on_device(logits, temperatures, uniforms)
-        return LaunchedStep(tokens, {id(w.seq): k for k, w in enumerate(sampling)}, sampling)
+        return LaunchedStep(tokens, {id(w.seq): k for k, w in enumerate(sampling)}, sampling, self.runner)

@@ -19,7 +19,7 @@ import torch
 
 from ..config.engine_config import ADMISSION_MARGIN_BLOCKS, BLOCK_SIZE, EngineConfig
 from .executor import ModelExecutor
-from .model import TORCH_DTYPE, Model, load_model, random_model
+from .model import NAME_OF_DTYPE, TORCH_DTYPE, Model, load_model, random_model
 from .scheduler import EventKind, Request, Scheduler, StepResult
 
 
@@ -32,30 +32,37 @@ class GenerationResult:
 
 
 class Engine:
-    def __init__(self, model: Union[str, Model], dtype: str = "bfloat16", block_size: int = BLOCK_SIZE,
+    def __init__(self, model: Union[str, Model], dtype: Optional[str] = None, block_size: int = BLOCK_SIZE,
                  num_blocks: Optional[int] = None, max_num_seqs: Optional[int] = None,
                  max_num_batched_tokens: Optional[int] = None,
                  admission_margin_blocks: int = ADMISSION_MARGIN_BLOCKS, record_logits: bool = False,
                  device: str = "cuda:0", kv_bytes: Optional[int] = None, fill_hbm: Optional[float] = None,
                  num_state_slots: Optional[int] = None) -> None:
-        """`model`: a folder, or a built `Model`.  The pool: `num_blocks` pages in every cache
-        group (default 3,584), or `kv_bytes` for the whole cache, or `fill_hbm`, the share of
-        the device memory still free once the weights are in place."""
+        """`model`: a folder, or a built `Model`.  `dtype`: "bfloat16" or "float32"; None takes the
+        folder's own (`torch_dtype` of its config.json), or the built model's.  The pool: `num_blocks`
+        pages in every cache group (default 3,584), or `kv_bytes` for the whole cache, or `fill_hbm`,
+        the share of the device memory still free once the weights are in place."""
+        if isinstance(model, str):
+            model = load_model(model, dtype, device)
+        if dtype is None:
+            dtype = NAME_OF_DTYPE[model.dtype]
         self.config = EngineConfig(dtype=dtype, block_size=block_size, num_blocks=num_blocks, kv_bytes=kv_bytes,
                                    fill_hbm=fill_hbm, admission_margin_blocks=admission_margin_blocks,
                                    max_num_seqs=max_num_seqs, max_num_batched_tokens=max_num_batched_tokens,
                                    num_state_slots=num_state_slots, device=device)
-        self.model = load_model(model, dtype, device) if isinstance(model, str) else model
+        self.model = model
         if self.model.dtype != TORCH_DTYPE[dtype]:
             raise ValueError(f"the engine was asked for {dtype} but the model it was given computes in {self.model.dtype}")
         self.num_blocks = self.config.pages(self.model.page_bytes(block_size), self._free_device_bytes)
-        self.cache = self.model.new_cache(block_size, self.num_blocks, self.config.state_slots)
+        keeps_state = any(spec is not None for spec in self.model.cache_specs()[1])
+        self.cache = self.model.new_cache(block_size, self.num_blocks,
+                                          self.config.state_slots_for(self.num_blocks, keeps_state))
         self.executor = ModelExecutor(self.model, self.cache)
         self.record_logits = record_logits
         self.scheduler = self._new_scheduler()
 
     @classmethod
-    def from_random(cls, config, seed: int = 0, dtype: str = "bfloat16", device: str = "cuda:0",
+    def from_random(cls, config, seed: int = 0, dtype: Optional[str] = None, device: str = "cuda:0",
                     std: float = 0.02, norm_std: float = 0.0, **engine_options) -> "Engine":
         """An engine over random weights drawn on the device from `seed` (no folder is written);
         `config` is a config.json dict or a typed config."""

@@ -27,6 +27,19 @@ from ..weights.loader import load_weights
 from ..weights.random_init import RandomWeights
 
 TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+NAME_OF_DTYPE = {v: k for k, v in TORCH_DTYPE.items()}
+
+
+def default_dtype(config) -> str:
+    """The precision a model computes in when the caller names none: what its config.json says
+    under `torch_dtype`, if that is one of the two the engine computes in; checkpoints stored in any
+    other type (float16, say) are served in bfloat16."""
+    stored = str(getattr(config, "torch_dtype", "") or "").replace("torch.", "")
+    return stored if stored in TORCH_DTYPE else "bfloat16"
+
+
+def plan_has_stops(plan: ModelPlan) -> bool:
+    return len(plan.schedule) > 0
 
 
 def _blocks_of(plan: ModelPlan, dtype, device):
@@ -60,8 +73,7 @@ class Model:
         return expected_tensors(self.plan)
 
     def optional_tensors(self) -> Tuple[str, ...]:
-        # a file of a model with a tied head may still store the head
-        return ("lm_head.weight",) if self.plan.head_name is None else ()
+        return tuple(self.plan.optional_names)
 
     def bind(self, weights: Mapping[str, torch.Tensor]) -> None:
         plan = self.plan
@@ -123,6 +135,28 @@ class Model:
         paged, states = self.cache_specs()
         return CacheManager(paged, states, block_size, num_blocks, num_slots, self.dtype, str(self.device))
 
+    def decode_fusable(self, ctx: StepContext) -> bool:
+        """Whether this step's blocks can run as one decode program: every sequence brings one token,
+        and every scheduled block, and the final norm that takes over from the last, says it launches
+        recordable kernels only at this many rows."""
+        rows, bs = ctx.num_tokens, ctx.cache.block_size
+        if rows != ctx.num_seqs or not plan_has_stops(self.plan):
+            return False
+        blocks = {entry.layer for entry in self.plan.schedule}
+        return (all(getattr(self.blocks[i], "decode_fusable", lambda *_: False)(rows, bs) for i in blocks)
+                and getattr(self.final_norm, "folded_for", lambda _: None)(rows) is not None)
+
+    def max_program_phases(self) -> int:
+        return 8 * len(self.plan.schedule) + 8
+
+    def _run_blocks(self, ctx: StepContext, stream: ResidualStream, first_norms) -> None:
+        for index, entry in enumerate(self.plan.schedule):
+            ctx.entry = index
+            ctx.cache_entry = index if entry.cache_from is None else entry.cache_from
+            ctx.writes_cache = entry.cache_from is None
+            stream.next_norm = first_norms[index + 1]
+            self.blocks[entry.layer].forward(ctx, stream)
+
     # ------------------------------------------------------------------ forward
     def forward(self, ctx: StepContext, token_ids: torch.Tensor, logit_rows: torch.Tensor) -> torch.Tensor:
         """Run `token_ids` (int32 [T]) through the schedule once; float32 logits
@@ -134,24 +168,25 @@ class Model:
         stream = ResidualStream(residual)
         # the norm that reads the stream first at every stop (and the final norm after the last)
         first_norms = [getattr(self.blocks[entry.layer], "mixer_norm", None) for entry in plan.schedule] + [self.final_norm]
-        fold = getattr(first_norms[0], "folded", None)
-        first_mixer = getattr(self.blocks[plan.schedule[0].layer], "mixer", None) if plan.schedule else None
-        if (self.dtype == torch.bfloat16 and fold is not None and 0 < T <= K.FOLD_MAX_ROWS and H % 8 == 0
-                and getattr(first_mixer, "takes_owed_rows", False)):
-            # few rows: the first norm is paid by the first product (see parts.OwedRows)
-            weight, eps = fold()
+        entry_fold = getattr(self.blocks[plan.schedule[0].layer], "entry_fold", None) if plan.schedule and T else None
+        fold = entry_fold(T) if entry_fold is not None else None
+        if fold is not None:
+            # the first block's norm lets the embedding prepare its rows (see parts.OwedRows)
+            norm, weight, eps = fold
             rows = torch.empty((T, H), dtype=torch.bfloat16, device=self.device)
             stats = torch.empty((T, K.stat_tiles(H)), dtype=torch.float32, device=self.device)
             K.embedding_rows(residual, self.embedding, token_ids, plan.embedding_scale, rows, weight, stats)
-            stream.owed, stream.owed_to = OwedRows(rows, stats, eps), first_norms[0]
+            stream.owed, stream.owed_to = OwedRows(rows, stats, eps), norm
         else:
             K.embedding(residual, self.embedding, token_ids, plan.embedding_scale)
-        for index, entry in enumerate(plan.schedule):
-            ctx.entry = index
-            ctx.cache_entry = index if entry.cache_from is None else entry.cache_from
-            ctx.writes_cache = entry.cache_from is None
-            stream.next_norm = first_norms[index + 1]
-            self.blocks[entry.layer].forward(ctx, stream)
+        program = ctx.program if fold is not None and self.decode_fusable(ctx) else None
+        if program is not None:
+            # every block's kernels become phases of one resident kernel, which runs when all are recorded
+            with K.recording(program):
+                self._run_blocks(ctx, stream, first_norms)
+            program.launch()
+        else:
+            self._run_blocks(ctx, stream, first_norms)
         rows = logit_rows.numel()
         if rows == 0:
             return torch.empty((0, plan.vocab_size), dtype=torch.float32, device=self.device)
@@ -162,12 +197,15 @@ class Model:
         return logits
 
 
-def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") -> Model:
+def load_model(model_dir: str, dtype: Optional[str] = None, device: str = "cuda:0") -> Model:
     """The model of a folder with config.json and safetensors weights; the class
-    of model is chosen by config.json's `architectures`."""
+    of model is chosen by config.json's `architectures`, and so is the precision if `dtype` is None
+    (`default_dtype`)."""
+    config = read_config(model_dir)
+    if dtype is None:
+        dtype = default_dtype(config)
     if dtype not in TORCH_DTYPE:
         raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
-    config = read_config(model_dir)
     model = Model(config.plan(), TORCH_DTYPE[dtype], device)
     model.config = config
     weights = load_weights(model_dir, model.expected_tensors(), model.optional_tensors())
@@ -175,16 +213,18 @@ def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") 
     return model
 
 
-def random_model(config, seed: int = 0, dtype: str = "bfloat16", device: str = "cuda:0", std: float = 0.02,
+def random_model(config, seed: int = 0, dtype: Optional[str] = None, device: str = "cuda:0", std: float = 0.02,
                  norm_std: float = 0.0) -> Model:
     """A model of `config` (a config.json dict, or a registered architecture's typed config) with
     random weights drawn on the device, tensor by tensor as the parts bind them: nothing is written
     to disk and no tensor exists twice, so the 72B shape's 145 GB fit one GPU.  The reference draws
     random weights only for its tiny test model (tests/tiny_model.py:21-50)."""
-    if dtype not in TORCH_DTYPE:
-        raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
     if isinstance(config, Mapping):
         config = read_config_dict(config)
+    if dtype is None:
+        dtype = default_dtype(config)
+    if dtype not in TORCH_DTYPE:
+        raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
     model = Model(config.plan(), TORCH_DTYPE[dtype], device)
     model.config = config
     model.bind(RandomWeights(model.expected_tensors(), seed, std, norm_std, device))

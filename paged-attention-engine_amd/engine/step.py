@@ -36,8 +36,9 @@ class StepEntry:
 class _CapturedStep:
     """A decode step recorded as a HIP graph: static inputs, the graph, its logits."""
 
-    def __init__(self, inputs: torch.Tensor) -> None:
+    def __init__(self, inputs: torch.Tensor, program=None) -> None:
         self.inputs = inputs
+        self.program = program  # room for the step's layers as one resident kernel (made before the recording)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
 
@@ -67,7 +68,8 @@ class StepRunner:
     TABLE_ROUND = 64    # block tables of captured steps are padded to a multiple of this many pages
     MAX_GRAPHS = 24
 
-    def __init__(self, model: Model, cache: CacheManager, use_graphs: bool = True) -> None:
+    def __init__(self, model: Model, cache: CacheManager, use_graphs: bool = True,
+                 use_programs: Optional[bool] = None) -> None:
         self.model = model
         self.cache = cache
         self.device = model.device
@@ -78,6 +80,16 @@ class StepRunner:
         self._graphs: Dict[tuple, _CapturedStep] = {}
         self.graph_replays = 0
         self.graph_recordings = 0
+        # Decode steps of a few rows can run their layers as one resident kernel where the model's parts
+        # allow it (see kernels.lib.DecodeProgram): the same bits as the separate kernels.  It is off
+        # unless asked for (`use_programs=True`, or PAE_DECODE_PROGRAMS=1): at the sizes measured the
+        # barrier between its phases costs what a kernel boundary costs, and the step is slower.
+        if use_programs is None:
+            use_programs = os.environ.get("PAE_DECODE_PROGRAMS", "0") == "1"
+        self.use_programs = bool(use_programs) and model.dtype == torch.bfloat16
+        self.program_groups: Optional[int] = None  # workgroups of a program; None: one per compute unit
+        self._eager_program = None
+        self._programs: List = []
         # a slow check for tests and debugging: after every step, wait for the device and see that the
         # products' ticket counters are back at zero
         self.check_tickets = bool(os.environ.get("PAE_CHECK_TICKETS"))
@@ -87,6 +99,19 @@ class StepRunner:
         self._staging_turn = 0
 
     STAGING_BUFFERS = 4
+
+    def _new_program(self):
+        if not self.use_programs:
+            return None
+        program = K.DecodeProgram(self.device, self.model.max_program_phases(), self.program_groups)
+        self._programs.append(program)
+        return program
+
+    def check_programs(self) -> None:
+        """Raise if any decode program of this runner was abandoned at a barrier.  The device must
+        have been waited for (a caller that holds the step's tokens has)."""
+        for program in self._programs:
+            program.check()
 
     def _to_device(self, flat: array, dst: Optional[torch.Tensor]) -> torch.Tensor:
         """A step's metadata to the device: into one of a few pinned buffers that take turns, and from
@@ -218,8 +243,12 @@ class StepRunner:
                     # the recording that has gone unused the longest goes; a step launched from it
                     # may still be running
                     torch.cuda.current_stream().synchronize()
-                    self._graphs.pop(next(iter(self._graphs)))
-                captured = _CapturedStep(torch.empty(len(flat), dtype=torch.int32, device=self.device))
+                    dropped = self._graphs.pop(next(iter(self._graphs)))
+                    if dropped.program is not None:
+                        dropped.program.check()
+                        self._programs.remove(dropped.program)
+                captured = _CapturedStep(torch.empty(len(flat), dtype=torch.int32, device=self.device),
+                                         self._new_program())
             self._graphs[key] = captured  # last used, last to go
             dev = self._to_device(flat, captured.inputs)
         else:
@@ -245,14 +274,21 @@ class StepRunner:
         for group, width in zip(cache.groups, widths):
             block_tables[group.index] = take(S * width).view(S, width)
 
+        program = None
+        if self.use_programs and T == S:
+            if captured is not None:
+                program = captured.program
+            else:  # a step launched kernel by kernel: one program serves them all, one after the other
+                program = self._eager_program = self._eager_program or self._new_program()
         ctx = StepContext(dtype=self.model.dtype, device=self.device, num_tokens=T, num_seqs=S,
                           positions=d_pos, tok_seq=d_seq, block_tables=block_tables, slots=d_slots,
                           cache=cache, seq_ids=seq_ids, q_starts=q_starts, q_lens=q_lens,
-                          past_lens=past_lens, host_slots=slots, memo=memo)
+                          past_lens=past_lens, host_slots=slots, memo=memo, program=program)
         if captured is None:
             logits = self.model.forward(ctx, d_ids, d_rows)
             if self.check_tickets:
                 K.check_tickets_zero(self.device)
+                self.check_programs()
             return logits
         if captured.graph is None:
             # record the step: nothing runs during the recording, so replay it right away
@@ -267,4 +303,5 @@ class StepRunner:
         self.graph_replays += 1
         if self.check_tickets:
             K.check_tickets_zero(self.device)
+            self.check_programs()
         return captured.logits[:R]

@@ -59,6 +59,7 @@ class TraceReplayer:
             out = self.runner.run(entries)
             if out.shape[0]:
                 logits = out.cpu().numpy()
+                self.runner.check_programs()
             for entry in entries:
                 self.cache.release_passed(entry.seq_id)
         for rid in record.get("end", []):

@@ -22,8 +22,11 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(_HERE), "csrc")
 LIB_NAME = f"libpae_{ARCH}.so"
 # Packed float32 instructions are switched off for every kernel: scalar float
-# code must compile to scalar float instructions.
-HIPCC_FLAGS = [f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17",
+# code must compile to scalar float instructions.  So is the contraction of a multiply and an add
+# into one fused instruction at the compiler's discretion: the same expression must round the same
+# way in every kernel it is compiled into (a step's layers run either as separate kernels or as
+# phases of one, and give the same bits); where a fused multiply-add is wanted it is written (fmaf).
+HIPCC_FLAGS = [f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 

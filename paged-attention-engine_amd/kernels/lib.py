@@ -10,6 +10,7 @@ functions raise.
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 from typing import Optional
 
@@ -32,7 +33,8 @@ def library():
     """The loaded kernel library (built at the first call if necessary)."""
     global _lib
     if _lib is None:
-        path = ensure_built()
+        # PAE_KERNEL_LIBRARY: a library built by hand from the same sources (a variant under measurement)
+        path = os.environ.get("PAE_KERNEL_LIBRARY") or ensure_built()
         try:
             lib = ctypes.CDLL(path)
         except OSError as err:
@@ -71,9 +73,19 @@ def _declare(lib) -> None:
         "pae_sample_chunks": [I],
         "pae_sample_static": [P, P, L, P, P, I, I, P],
         "pae_sample_static_slots": [],
+        "pae_sample_static_prepare": [],
         "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, P, P, P],
         "pae_attn_decode_split": [],
         "pae_attn_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
+        "pae_program_phase_bytes": [],
+        "pae_program_barrier_bytes": [],
+        "pae_program_max_rows": [],
+        "pae_program_max_groups": [],
+        "pae_program_put_product": [P, I, I, P, L, P, L, P, P, I, I, I, I, I, P, P, P, I, F, P, L, P, I, P, P],
+        "pae_program_put_product_rope": [P, I, P, L, P, L, P, P, I, I, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P, P, P,
+                                         I, F],
+        "pae_program_put_attention": [P, I, P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, P, P, P],
+        "pae_program_run": [P, I, P, P, I, I, I, P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -134,6 +146,7 @@ def device_arch() -> str:
 
 def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> None:
     """out[t] = scale * table[ids[t]] as float32; ids int32 (checked against the table by the caller)."""
+    _not_while_recording("embedding")
     _gpu(out, table, ids)
     T, H = out.shape
     assert out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous()
@@ -144,6 +157,7 @@ def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: 
 
 def logits_finish(logits: torch.Tensor, scale: float = 1.0, softcap: float = 0.0) -> None:
     """In place: logits = scale * logits, then with a soft cap c > 0, c * tanh(logits / c)."""
+    _not_while_recording("logits_finish")
     _gpu(logits)
     assert logits.dtype == torch.float32 and logits.is_contiguous()
     _check(library().pae_logits_finish(logits.data_ptr(), logits.numel(), float(scale), float(softcap), _stream()))
@@ -156,6 +170,7 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     `delta` is the pending branch output: [T, H] in out's dtype, or float32 partial sums
     [P, T, H] that are added in order.  With `rows` (int32), out[b] comes from source row
     rows[b] and nothing is written back."""
+    _not_while_recording("add_rmsnorm")
     _gpu(residual, delta, weight, out, rows)
     H = residual.shape[-1]
     n = out.shape[0]
@@ -181,6 +196,7 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
 
 
 def residual_add(residual: torch.Tensor, delta: torch.Tensor) -> None:
+    _not_while_recording("residual_add")
     _gpu(residual, delta)
     assert residual.dtype == torch.float32 and residual.shape == delta.shape
     assert residual.is_contiguous() and delta.is_contiguous()
@@ -191,6 +207,7 @@ def residual_add(residual: torch.Tensor, delta: torch.Tensor) -> None:
 def copy_int32_from_pinned(dst: torch.Tensor, src: torch.Tensor, n: int) -> None:
     """dst[:n] = src[:n] by a kernel on the current stream; `src` is pinned host memory (which the
     GPU reads in place) and must stay as it is until the kernel has run."""
+    _not_while_recording("copy_int32_from_pinned")
     _gpu(dst)
     assert dst.dtype == torch.int32 == src.dtype and dst.is_contiguous() and src.is_contiguous()
     assert src.is_pinned() and 0 <= n <= min(dst.numel(), src.numel())
@@ -200,6 +217,7 @@ def copy_int32_from_pinned(dst: torch.Tensor, src: torch.Tensor, n: int) -> None
 def scatter_int32(dst: torch.Tensor, dst_idx: torch.Tensor, src: torch.Tensor, src_idx: torch.Tensor, n: int) -> None:
     """dst[dst_idx[i]] = src[src_idx[i]] for i < n (int32 everywhere; the index lists may be longer than n).
     The caller vouches for the indices: they are not checked on the device."""
+    _not_while_recording("scatter_int32")
     _gpu(dst, dst_idx, src, src_idx)
     for t in (dst, dst_idx, src, src_idx):
         assert t.dtype == torch.int32 and t.is_contiguous()
@@ -233,6 +251,7 @@ def rope_kv_write(qkv: torch.Tensor, nh: int, nkv: int, hd: int, rot: int, cos_s
     into their cache slots (skipped when `k_cache` is None: then the row holds query heads only
     and nkv must be 0).  With `bias` (one value per feature of the row) the row stands for the
     projection without its bias, which is added here first."""
+    _not_while_recording("rope_kv_write")
     _gpu(qkv, cos_sin, positions, tok_seq, block_tables, k_cache, v_cache, bias)
     if bias is not None:
         assert bias.numel() == (nh + 2 * nkv) * hd
@@ -269,10 +288,125 @@ def kv_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, positions: torch.Ten
 def swiglu(out: torch.Tensor, x: torch.Tensor, block: int = 0) -> None:
     """out[t, j] = silu(gate_j) * up_j for x of width 2 I: gate = x[:, :I], up = x[:, I:], or,
     with `block` > 0, blocks of `block` gate features each followed by their up features."""
+    _not_while_recording("swiglu")
     _gpu(out, x)
     T, I = out.shape
     assert x.shape == (T, 2 * I) and x.dtype == out.dtype and x.is_contiguous() and out.is_contiguous()
     _check(library().pae_swiglu(code_of(x.dtype), out.data_ptr(), x.data_ptr(), T, I, block, _stream()))
+
+
+# ---------------------------------------------------------------------------------- decode programs
+# A decode step's products and attention as one resident kernel (csrc/decode_program.hip).  While a
+# program is recording, `gemm_skinny`, `gemm_skinny_rope` and `attn_decode` append a phase to it
+# instead of launching; `rope_table`, which reads the step's positions only, runs at once; every other
+# wrapper refuses.  `launch()` then runs the phases in the order they were recorded, each after the
+# one before it has finished everywhere, as the separate launches would.
+_RECORDING = None
+PROGRAM_SPIN_LIMIT = 2_000_000  # polls of a barrier before a workgroup gives up (about two seconds)
+
+
+def _not_while_recording(name: str) -> None:
+    if _RECORDING is not None:
+        raise KernelError(f"{name} cannot be a phase of a decode program; a part that calls it must not say it is fusable")
+
+
+def program_max_rows() -> int:
+    return library().pae_program_max_rows()
+
+
+_PROGRAM_BARRIERS: dict = {}  # (device index, workgroups) -> zeroed barrier block
+
+
+class DecodeProgram:
+    """Room for a list of phases (in pinned host memory, where it is written, and on the device, where
+    the kernel reads it) and what running them needs.  A program recorded into a HIP graph keeps its
+    list for as long as the graph lives: every replay copies it to the device again."""
+
+    def __init__(self, device, max_phases: int, groups: Optional[int] = None) -> None:
+        lib = library()
+        self.device = torch.device(device)
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("a decode program's buffers must exist before a graph is recorded")
+        with torch.cuda.device(self.device):
+            most = lib.pae_program_max_groups()
+        if most < 1:
+            _check(most)
+        self.groups = most if groups is None else int(groups)
+        if not 1 <= self.groups <= most:
+            raise KernelError(f"{self.groups} workgroups cannot all be resident (at most {most})")
+        self.phase_bytes = lib.pae_program_phase_bytes()
+        self.max_phases = max_phases
+        ints = self.phase_bytes * max_phases // 4
+        self.host = torch.zeros(ints, dtype=torch.int32, pin_memory=True)
+        self.on_device = torch.zeros(ints, dtype=torch.int32, device=self.device)
+        self.error = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        key = (self.device.index or 0, self.groups)
+        if key not in _PROGRAM_BARRIERS:
+            _PROGRAM_BARRIERS[key] = torch.zeros(lib.pae_program_barrier_bytes() // 4, dtype=torch.int32, device=self.device)
+        self.barrier = _PROGRAM_BARRIERS[key]
+        skinny_tickets(self.device)
+        self.host_ptr = self.host.data_ptr()
+        self.count = 0
+        self.quad_lds = 0
+        self.keep: list = []
+        self._read: Optional[torch.cuda.Event] = None
+
+    def begin(self) -> None:
+        if self._read is not None:
+            self._read.synchronize()  # the launch before has copied the list to the device
+        self.count, self.quad_lds, self.keep = 0, 0, []
+
+    def add(self, code: int, *tensors) -> None:
+        """`code`: what a pae_program_put_* call returned (the bytes of LDS a quad needs, or an error)."""
+        if code < 0:
+            _check(code)
+        if self.count + 1 > self.max_phases:
+            raise KernelError(f"a decode program of more than {self.max_phases} phases")
+        self.count += 1
+        self.quad_lds = max(self.quad_lds, code)
+        self.keep.append(tensors)  # what the phase reads and writes stays alive until the program has run
+
+    def launch(self) -> None:
+        if self.count == 0:
+            return
+        global _RECORDING
+        assert _RECORDING is None, "a program is launched after its recording has ended"
+        copy_int32_from_pinned(self.on_device, self.host, self.count * self.phase_bytes // 4)
+        _check(library().pae_program_run(self.on_device.data_ptr(), self.count, self.barrier.data_ptr(),
+                                         self.error.data_ptr(), self.groups, self.quad_lds, PROGRAM_SPIN_LIMIT, _stream()))
+        if not torch.cuda.is_current_stream_capturing():
+            self._read = self._read or torch.cuda.Event()
+            self._read.record()
+
+    def check(self) -> None:
+        """Raise if a launch of this program gave up at a barrier (call after the device has been waited for)."""
+        code = int(self.error[0])
+        if code:
+            self.error[0] = 0
+            self.barrier.zero_()
+            skinny_tickets(self.device).zero_()
+            raise KernelError(f"the decode program's workgroups did not all arrive at the barrier after phase {code - 1}: "
+                              "the program was abandoned and its results are invalid")
+
+
+class recording:
+    """`with recording(program):` the product and decode-attention wrappers append phases to `program`."""
+
+    def __init__(self, program: DecodeProgram) -> None:
+        self.program = program
+
+    def __enter__(self):
+        global _RECORDING
+        if _RECORDING is not None:
+            raise KernelError("a decode program is already recording")
+        self.program.begin()
+        _RECORDING = self.program
+        return self.program
+
+    def __exit__(self, *exc):
+        global _RECORDING
+        _RECORDING = None
+        return False
 
 
 SKINNY_MAX_ROWS = 64
@@ -301,6 +435,7 @@ def embedding_rows(residual: torch.Tensor, table: torch.Tensor, ids: torch.Tenso
     """`embedding` for a step whose first norm is folded into the products: beside residual[t] =
     scale * table[ids[t]], next_rows[t] = bfloat16(residual[t] * next_w) and next_stats[t][j] = the sum
     of squares of residual[t] over columns 16 j .. 16 j + 15."""
+    _not_while_recording("embedding_rows")
     _gpu(residual, table, ids, next_rows, next_w, next_stats)
     T, H = residual.shape
     assert residual.dtype == torch.float32 and residual.is_contiguous() and table.is_contiguous()
@@ -316,6 +451,7 @@ def embedding_rows(residual: torch.Tensor, table: torch.Tensor, ids: torch.Tenso
 
 def scaled_rows(rows: torch.Tensor, stats: torch.Tensor, eps: float) -> torch.Tensor:
     """rows[m] * rsqrt(sum(stats[m]) / width + eps) as bfloat16: rows whose scale was owed, paid."""
+    _not_while_recording("scaled_rows")
     _gpu(rows, stats)
     M, H = rows.shape
     assert rows.dtype == torch.bfloat16 and rows.is_contiguous()
@@ -364,21 +500,18 @@ def skinny_splits(N: int, K: int, M: int = 1) -> int:
     return -(-K // k_per)
 
 
-def residual_splits(N: int, K: int, M: int) -> int:
-    """k ranges for a product of up to 16 rows that adds itself into the residual (EPI_RESIDUAL).  One
-    range runs as sixteen wavefronts a workgroup that share out k, with no tickets and no trip to memory
-    for partial sums, and is ahead wherever the 16-row workgroups fill the chip or have little to read
-    (1.5B O at 8 rows 7.2 -> 5.9 us, 7B down 38.3 -> 36.1 us, 72B down 111 -> 107.5 us); a few workgroups
-    with much to read each want ranges (1.5B down: 96 workgroups of 287 KB, 17.4 us in one range, 12.5 in five).
-    From 9 rows on the kernels for many rows are there as well, and their ranges are ahead where they are
-    more than two (at 16 rows: 7B down 42.7 us in one range, 33.2 in eight; 72B down 130 and 92)."""
-    if M > 8:
-        many = skinny_splits(N, K, M)
-        return many if many > 2 else 1
+def residual_splits(N: int, K: int, M: int = 1) -> int:
+    """k ranges for a product of up to 16 rows that adds itself into the residual (EPI_RESIDUAL), from
+    the product's sizes alone: a row's sums are the same bits whatever it is batched with, launched by
+    itself or as a phase of a decode program.  Four ranges run side by side in one workgroup of sixteen
+    wavefronts, with no tickets and no trip to memory for partial sums, and are ahead wherever the 16-row
+    workgroups fill the chip or have little to read (1.5B O at 8 rows 7.2 -> 5.9 us, 7B down 38.3 -> 36.1
+    us, 72B down 111 -> 107.5 us); a few workgroups with much to read each want ticketed ranges (1.5B
+    down: 96 workgroups of 287 KB, 17.4 us in one workgroup each, 12.5 in five ranges)."""
     tiles = -(-N // 16)
-    if tiles >= 192 or 32 * K <= 65536:
-        return 1
-    return skinny_splits(N, K, M)
+    if K >= 1024 and (tiles >= 192 or 32 * K <= 65536):
+        return -(-K // (-(-(-(-K // 4)) // 128) * 128))  # four, as the rounding to 128 leaves them
+    return skinny_splits(N, K, 1)
 
 
 def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -421,11 +554,46 @@ def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optio
     bp, bf = _param(bias)
     sp, st, se = _row_scale(row_scale, M, K_)
     parts, counters = _ticket_scratch(a.device, M, N, splits if epilogue != EPI_F32 else 1)
+    if _RECORDING is not None:
+        _RECORDING.add(library().pae_program_put_product(
+            _RECORDING.host_ptr, _RECORDING.count, epilogue, out.data_ptr(), out.stride(-2), a.data_ptr(), a.stride(0),
+            w.data_ptr(), bp, bf, M, N, K_, splits, _ptr(parts), _ptr(counters), sp, st, se, nr, ld_next, nw, nwf, ns,
+            None), out, a, w, bias, parts, row_scale, following)
+        return
+    checking = (parts is not None and CHECK_TICKET_SUMS and not torch.cuda.is_current_stream_capturing())
+    before = out.clone() if checking and epilogue == EPI_RESIDUAL else None
     _launch_ticketed(counters, lambda: library().pae_gemm_skinny(
         epilogue, out.data_ptr(), out.stride(-2), a.data_ptr(), a.stride(0), w.data_ptr(), bp, bf, M, N, K_, splits,
         M * N, _ptr(parts), _ptr(counters), sp, st, se, nr, ld_next, nw, nwf, ns, _stream()))
+    if checking:
+        _check_ticket_sums(out, before, a, w, bias, epilogue, splits, row_scale, following)
 
 
+# PAE_CHECK_TICKETS=sums: every product whose k ranges are added up inside the kernel is computed a
+# second time in one k range (no tickets, no partial sums in memory) and the two results are compared.
+# A partial sum read stale (from an earlier launch, or before it had arrived) is a whole k range's worth
+# of error and shows far above the difference that the other order of adding leaves.
+CHECK_TICKET_SUMS = os.environ.get("PAE_CHECK_TICKETS", "") == "sums"
+
+
+def _check_ticket_sums(out, before, a, w, bias, epilogue, splits, row_scale, following) -> None:
+    again = before if before is not None else torch.empty_like(out)
+    follow = None
+    if following is not None:
+        follow = (torch.empty_like(following[0]), following[1], torch.empty_like(following[2]))
+    pairs = [(out, again)] + ([(following[0], follow[0])] if follow is not None else [])
+    gemm_skinny(again, a, w, bias, epilogue, 1, row_scale, follow)
+    for got, want in pairs:
+        got, want = got.float(), want.float()
+        bound = 2.0 ** -6 * float(want.abs().max()) + 1e-30
+        worst = float((got - want).abs().max())
+        if not worst <= bound:
+            raise KernelError(f"a product of {tuple(a.shape)} by {tuple(w.shape)} added up over {splits} k ranges inside "
+                              f"the kernel differs from the same product in one range by {worst:.3e} (bound {bound:.3e}): "
+                              "a partial sum was read before it had arrived, or left over from another launch")
+
+
+TICKET_ARCHS = ("gfx950",)  # chips on which the fence-free ticket scheme has been validated
 _TICKETS: dict = {}        # device index -> counters
 _TICKET_STREAM: dict = {}  # device index -> the stream whose launches use them
 
@@ -441,6 +609,11 @@ def skinny_tickets(device) -> torch.Tensor:
     if index not in _TICKETS:
         if torch.cuda.is_current_stream_capturing():
             raise KernelError("the ticket counters must exist before a graph is recorded")
+        if device_arch() not in TICKET_ARCHS:
+            # the scheme leans on how this chip's device-scope stores and loads reach the memory side
+            # (see SkinnyTickets in csrc/gemm_skinny.hip); it has been validated on these chips only
+            raise KernelError(f"k ranges added up inside a kernel are validated on {', '.join(TICKET_ARCHS)} only, "
+                              f"not on {device_arch()}")
         _TICKETS[index] = torch.zeros(1 << 16, dtype=torch.int32, device=device)
         _TICKET_STREAM[index] = torch.cuda.current_stream(device).cuda_stream
     return _TICKETS[index]
@@ -493,8 +666,9 @@ def whole_sum_splits(N: int, K: int, M: int) -> int:
       14B 37 -> 31 us in four, 72B 87 -> 54 us in six);
     * not with very few weight rows, where the rows of activations are shared out instead."""
     tiles, groups = -(-N // 32), -(-N // 128)
-    if M <= 8:
-        # long rows of weights and not so many of them that the chip is full many times over (the QKV
+    if M <= FOLD_MAX_ROWS:
+        # from the sizes alone, so that a row's sums do not depend on the batch (as `residual_splits`).
+        # Long rows of weights and not so many of them that the chip is full many times over (the QKV
         # product of the 72B sizes): ranges of about 2,048 (at 8 rows 42.6 -> 40.4 us in four, at one row 39 -> 37 us)
         return max(1, min(4, K // 2048)) if N <= 16384 else 1
     if 128 <= groups < 256:
@@ -545,6 +719,13 @@ def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias
     splits = 1 if splits is None else splits
     parts, counters = _ticket_scratch(a.device, M, N, splits)
     sp, st, se = _row_scale(row_scale, M, K_)
+    if _RECORDING is not None:
+        _RECORDING.add(lib.pae_program_put_product_rope(
+            _RECORDING.host_ptr, _RECORDING.count, q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0),
+            w.data_ptr(), bp, bf, M, K_, nh, nkv, hd, rot, _ptr(cos_sin) if rot else None, positions.data_ptr(),
+            _ptr(tok_seq), _ptr(block_tables), max_blocks, block_size, _ptr(k_cache), _ptr(v_cache), splits, _ptr(parts),
+            _ptr(counters), sp, st, se), q_out, a, w, bias, cos_sin, parts, row_scale)
+        return
     _launch_ticketed(counters, lambda: lib.pae_gemm_skinny_rope(
         q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(), bp, bf, M, K_, nh, nkv, hd, rot,
         _ptr(cos_sin) if rot else None, positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks,
@@ -553,6 +734,7 @@ def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias
 
 def gemm_plain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:
     """out[M, N] = a[M, K] @ w[N, K]^T (+ bias), float32 accumulation in k order."""
+    _not_while_recording("gemm_plain")
     _gpu(out, a, w, bias)
     M, K = a.shape
     N = w.shape[0]
@@ -570,6 +752,7 @@ def paged_attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.T
                             nh: int, nkv: int, hd: int, scale: float, window: int) -> None:
     """out[t, h*hd:(h+1)*hd] = attention of query head h of token t over the cached
     keys start..positions[t] of sequence tok_seq[t]."""
+    _not_while_recording("paged_attention_generic")
     _gpu(out, q, k_cache, v_cache, positions, tok_seq, block_tables)
     T = q.shape[0]
     bs = k_cache.shape[2]
@@ -608,6 +791,16 @@ def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cac
     max_splits = -(-block_tables.shape[1] * bs // library().pae_attn_decode_split())
     part_acc = torch.empty((n * nh * max_splits, hd), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n * nh * max_splits, 2), dtype=torch.float32, device=q.device)
+    if _RECORDING is not None:
+        counters = skinny_tickets(q.device)
+        if n * nkv > counters.numel():
+            raise KernelError(f"{n} tokens by {nkv} key/value heads need more ticket counters than there are")
+        _RECORDING.add(library().pae_program_put_attention(
+            _RECORDING.host_ptr, _RECORDING.count, out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
+            k_cache.data_ptr(), v_cache.data_ptr(), dec_work.data_ptr(), n, block_tables.data_ptr(),
+            block_tables.shape[1], bs, nh, nkv, hd, float(scale), int(window), part_acc.data_ptr(), part_ml.data_ptr(),
+            counters.data_ptr()), out, q, part_acc, part_ml)
+        return
     _check(library().pae_attn_decode_bf16(
         out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
         dec_work.data_ptr(), n, block_tables.data_ptr(), block_tables.shape[1], bs, nh, nkv, hd, float(scale),
@@ -624,6 +817,7 @@ def attn_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_ca
     flat token, number of tokens <= PREFILL_TILE).  One workgroup per run and head, whose
     wavefronts share out the keys; workgroups start in the order of `tiles`, so the runs with
     the most keys should come first."""
+    _not_while_recording("attn_prefill")
     _gpu(out, q, k_cache, v_cache, tiles, positions, block_tables)
     bs = k_cache.shape[2]
     assert q.dtype == torch.bfloat16 == out.dtype == k_cache.dtype and q.stride(1) == 1 and out.stride(1) == 1
@@ -642,6 +836,7 @@ def sample(tokens: torch.Tensor, logits: torch.Tensor, temperature: Optional[tor
            uniform: Optional[torch.Tensor]) -> None:
     """tokens[r] = argmax(logits[r]) where temperature[r] == 0 (or no temperatures
     are given), else the inverse-CDF sample of softmax(logits[r] / temperature[r]) at uniform[r]."""
+    _not_while_recording("sample")
     _gpu(tokens, logits, temperature, uniform)
     R, V = logits.shape
     assert logits.dtype == torch.float32 and logits.stride(1) == 1
@@ -664,6 +859,7 @@ def sample_static(tokens: torch.Tensor, logits: torch.Tensor, temperature: Optio
     """`sample` without a workspace: the chunk results go to a buffer inside the library's image on
     the GPU, so nothing is allocated here or there.  Rows times chunks beyond that buffer's slots
     are refused; calls that overlap on one GPU race (they share the buffer)."""
+    _not_while_recording("sample_static")
     _gpu(tokens, logits, temperature, uniform)
     R, V = logits.shape
     assert logits.dtype == torch.float32 and logits.stride(1) == 1

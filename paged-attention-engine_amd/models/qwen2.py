@@ -166,6 +166,8 @@ class Qwen2Config:
             head_name=None if self.tie_word_embeddings else "lm_head.weight",
             final_norm_prefix="model.norm.",
             max_positions=self.max_position_embeddings,
+            # a file of a model with a tied head may still store the head
+            optional_names=("lm_head.weight",) if self.tie_word_embeddings else (),
         )
 
 

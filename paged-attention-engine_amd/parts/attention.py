@@ -70,6 +70,16 @@ class PagedAttention(Part):
     def graph_max_rows(self):
         return rows_a_graph_may_hold(self.dtype, self.spec.hidden_size, self.spec.num_heads * self.spec.head_dim)
 
+    def decode_fusable(self, rows: int, block_size: int) -> bool:
+        """One token a sequence, few rows: the fused projection, the decode attention and the output
+        product are all this mixer launches (a rotation that hands out its table runs inside the first)."""
+        s = self.spec
+        group = s.num_heads // s.num_kv_heads
+        return (self.dtype == torch.bfloat16 and 0 < rows <= K.program_max_rows() and self._matrix_cores(block_size)
+                and s.head_dim in (64, 128) and group * s.head_dim <= 1024 and not s.out_bias
+                and hasattr(self.position, "rotary_table") and s.hidden_size % 8 == 0
+                and getattr(s.position, "rotary_dim", 0) % 16 == 0)
+
     def paged_spec(self):
         return attention_pages(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)
 
@@ -85,28 +95,28 @@ class PagedAttention(Part):
 
     def tensors(self, prefix):
         s = self.spec
-        out = {prefix + "q_proj.weight": (s.num_heads * s.head_dim, s.hidden_size),
-               prefix + "k_proj.weight": (s.num_kv_heads * s.head_dim, s.hidden_size),
-               prefix + "v_proj.weight": (s.num_kv_heads * s.head_dim, s.hidden_size),
-               prefix + "o_proj.weight": (s.hidden_size, s.num_heads * s.head_dim)}
+        out = {prefix + s.q_name + ".weight": (s.num_heads * s.head_dim, s.hidden_size),
+               prefix + s.k_name + ".weight": (s.num_kv_heads * s.head_dim, s.hidden_size),
+               prefix + s.v_name + ".weight": (s.num_kv_heads * s.head_dim, s.hidden_size),
+               prefix + s.o_name + ".weight": (s.hidden_size, s.num_heads * s.head_dim)}
         if s.qkv_bias:
-            out[prefix + "q_proj.bias"] = (s.num_heads * s.head_dim,)
-            out[prefix + "k_proj.bias"] = (s.num_kv_heads * s.head_dim,)
-            out[prefix + "v_proj.bias"] = (s.num_kv_heads * s.head_dim,)
+            out[prefix + s.q_name + ".bias"] = (s.num_heads * s.head_dim,)
+            out[prefix + s.k_name + ".bias"] = (s.num_kv_heads * s.head_dim,)
+            out[prefix + s.v_name + ".bias"] = (s.num_kv_heads * s.head_dim,)
         if s.out_bias:
-            out[prefix + "o_proj.bias"] = (s.hidden_size,)
+            out[prefix + s.o_name + ".bias"] = (s.hidden_size,)
         return out
 
     def bind(self, prefix, weights):
         s = self.spec
-        names = ("q_proj", "k_proj", "v_proj")
+        names = (s.q_name, s.k_name, s.v_name)
         w = torch.cat([weights[prefix + n + ".weight"] for n in names], dim=0)
         b = (torch.cat([weights[prefix + n + ".bias"] for n in names], dim=0) if s.qkv_bias else None)
         self.qkv = Linear(self.matrix(w), None if b is None else self.vector(b))
         nq = s.num_heads * s.head_dim
         self.q_only = Linear(self.qkv.weight[:nq], None if b is None else self.qkv.bias[:nq])
-        ob = weights.get(prefix + "o_proj.bias") if s.out_bias else None
-        self.out = Linear(self.matrix(weights[prefix + "o_proj.weight"]), None if ob is None else self.vector(ob))
+        ob = weights[prefix + s.o_name + ".bias"] if s.out_bias else None
+        self.out = Linear(self.matrix(weights[prefix + s.o_name + ".weight"]), None if ob is None else self.vector(ob))
 
     def _project_encode_store(self, ctx, x, k_cache, v_cache, table):
         """Queries (and, at a stop that owns its cache, keys and values) of the step's tokens:
@@ -151,7 +161,8 @@ class PagedAttention(Part):
     def forward(self, ctx, x):
         """`x`: normalised activations, or `OwedRows` (the projection then pays their scale)."""
         s = self.spec
-        k_cache, v_cache = ctx.cache.kv_of(ctx.cache_entry)
+        pages = ctx.cache.pages_of(ctx.cache_entry)  # as declared in `paged_spec`
+        k_cache, v_cache = pages["k"], pages["v"]
         table = ctx.block_tables[ctx.cache.group_of(ctx.cache_entry)]
         qkv = self._project_encode_store(ctx, x, k_cache, v_cache, table)
         attn = torch.empty((x.shape[0], s.num_heads * s.head_dim), dtype=x.dtype, device=x.device)

@@ -24,6 +24,14 @@ from typing import Callable, Dict, List, Mapping, Optional, Tuple
 import torch
 
 
+class ScaleShape(tuple):
+    """The declared shape of a tensor that multiplies activations elementwise (a norm's weight).
+    Equal to the plain tuple; random mode reads `centre` and draws such a tensor about one instead
+    of about zero.  A part marks the tensor where it declares it, whatever the tensor is called."""
+
+    centre = 1.0
+
+
 class OwedRows:
     """Activations whose division by their root mean square is still owed.
 
@@ -81,14 +89,14 @@ class BranchSink:
     """Where a branch's last product may deliver itself instead of returning its output: added
     into the stream's residual in place, with the rows the following norm's consumer wants
     prepared on the way.  `norm` is the norm part that will read the stream next; it must offer
-    `folded() -> (weight, eps)` for the offer to be taken up."""
+    `folded_for(rows) -> (weight, eps) | None` for the offer to be taken up."""
 
     def __init__(self, stream: ResidualStream, norm) -> None:
         self.stream, self.norm = stream, norm
 
-    def folded(self):
-        fold = getattr(self.norm, "folded", None)
-        return fold() if fold is not None else None
+    def folded(self, rows: int):
+        fold = getattr(self.norm, "folded_for", None)
+        return fold(rows) if fold is not None else None
 
     def deliver(self, owed: OwedRows) -> None:
         self.stream.pending = None
@@ -136,6 +144,9 @@ class StepContext:
     cache_entry: int = 0               # the stop whose cache is read (entry itself unless it borrows)
     writes_cache: bool = True
     sink: Optional["BranchSink"] = None  # set by the block around a branch: see BranchSink
+    # room for the step's layers as one resident kernel (kernels.lib.DecodeProgram), offered by the step
+    # function for steps in which every sequence brings one token; None: every kernel is launched by itself
+    program: Optional[object] = None
     # what a part computes once per step for every layer that has the same part (a table of angles,
     # say), under a key of the part's choosing; the step function also leaves here, under
     # `step_lists_key`, the index lists a part asked for (`Part.step_lists`), as int32 device tensors
@@ -155,6 +166,13 @@ class Part:
     # True when `forward` takes its input as `OwedRows` as well as a plain tensor (the block
     # settles them for parts that do not).
     takes_owed_rows = False
+
+    def decode_fusable(self, rows: int, block_size: int) -> bool:
+        """Whether, in a step of `rows` sequences that bring one token each, `forward` does all of its
+        device work through wrappers that a decode program can record (see kernels.lib.recording):
+        the few-row products and the decode attention.  A part that launches anything else, or calls
+        the platform's libraries, must say no (the default)."""
+        return False
 
     def __init__(self, spec, dtype: torch.dtype, device) -> None:
         self.spec = spec

@@ -49,6 +49,17 @@ class PreNormBlock:
         for part, prefix in self._named():
             part.bind(prefix, weights)
 
+    def decode_fusable(self, rows: int, block_size: int) -> bool:
+        """Whether a step of `rows` single tokens runs this block through recordable kernels alone."""
+        return all(part.decode_fusable(rows, block_size) for part, _ in self._named())
+
+    def entry_fold(self, rows: int):
+        """(norm, weight, eps) if whatever fills the stream before this block (the embedding) may
+        prepare the first norm's rows for a step of `rows` rows; None if the norm runs its own kernel."""
+        fold = getattr(self.mixer_norm, "folded_for", None) if self.mixer.takes_owed_rows else None
+        got = fold(rows) if fold is not None else None
+        return None if got is None else (self.mixer_norm, *got)
+
     def forward(self, ctx, stream: ResidualStream) -> None:
         """Each branch is offered a sink: its last product may add itself into the residual and
         prepare the rows of the norm that reads the stream next (this block's second norm, then

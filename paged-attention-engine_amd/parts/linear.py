@@ -87,9 +87,9 @@ class Linear:
         prepares the following product's rows; nothing is returned then."""
         if x.dtype == torch.bfloat16 and self.bias is None and x.shape[0] and K.skinny_supported(x, self.weight):
             splits = K.skinny_splits(self.out_features, self.in_features, x.shape[0])
-            fold = sink.folded() if sink is not None else None
+            fold = sink.folded(x.shape[0]) if sink is not None else None
             residual = sink.stream.residual if sink is not None else None
-            if (fold is not None and x.shape[0] <= K.FOLD_MAX_ROWS and residual.dtype == torch.float32
+            if (fold is not None and residual.dtype == torch.float32
                     and residual.is_contiguous() and tuple(residual.shape) == (x.shape[0], self.out_features)):
                 weight, eps = fold
                 rows = torch.empty((x.shape[0], self.out_features), dtype=torch.bfloat16, device=x.device)

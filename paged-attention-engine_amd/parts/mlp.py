@@ -26,14 +26,15 @@ class SwiGLU(Part):
 
     def tensors(self, prefix):
         s = self.spec
-        return {prefix + "gate_proj.weight": (s.intermediate_size, s.hidden_size),
-                prefix + "up_proj.weight": (s.intermediate_size, s.hidden_size),
-                prefix + "down_proj.weight": (s.hidden_size, s.intermediate_size)}
+        return {prefix + s.gate_name + ".weight": (s.intermediate_size, s.hidden_size),
+                prefix + s.up_name + ".weight": (s.intermediate_size, s.hidden_size),
+                prefix + s.down_name + ".weight": (s.hidden_size, s.intermediate_size)}
 
     BLOCK = 8  # gate and up rows alternate in blocks of this many (the skinny product's gated epilogue)
 
     def bind(self, prefix, weights):
-        gate, up = weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]
+        s = self.spec
+        gate, up = weights[prefix + s.gate_name + ".weight"], weights[prefix + s.up_name + ".weight"]
         inter, hidden = gate.shape
         self.block = self.BLOCK if (self.dtype == torch.bfloat16 and inter % self.BLOCK == 0) else 0
         if self.block:
@@ -43,7 +44,12 @@ class SwiGLU(Part):
         else:
             gate_up = torch.cat([gate, up], dim=0)
         self.gate_up = Linear(self.matrix(gate_up))
-        self.down = Linear(self.matrix(weights[prefix + "down_proj.weight"]))
+        self.down = Linear(self.matrix(weights[prefix + s.down_name + ".weight"]))
+
+    def decode_fusable(self, rows: int, block_size: int) -> bool:
+        s = self.spec
+        return (self.dtype == torch.bfloat16 and bool(self.block) and 0 < rows <= K.program_max_rows()
+                and s.hidden_size % 8 == 0 and s.intermediate_size % 8 == 0)
 
     def forward(self, ctx, x):
         """`x`: normalised activations, or `OwedRows` (the gated product then pays their scale)."""

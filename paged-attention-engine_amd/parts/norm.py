@@ -13,21 +13,29 @@ from typing import Optional
 import torch
 
 from ..kernels import lib as K
-from .base import OwedRows, Part, ResidualStream, register_norm
+from .base import OwedRows, Part, ResidualStream, ScaleShape, register_norm
 
 
 @register_norm("rmsnorm")
 class RMSNorm(Part):
     graph_safe = True
     def tensors(self, prefix):
-        return {prefix + "weight": (self.spec.size,)}
+        return {prefix + self.spec.weight_name: ScaleShape((self.spec.size,))}
 
     def bind(self, prefix, weights):
-        self.weight = self.vector(weights[prefix + "weight"])
+        self.weight = self.vector(weights[prefix + self.spec.weight_name])
 
-    def folded(self):
-        """(weight, eps): what a product needs to prepare rows for this norm (see `OwedRows`)."""
+    def folded_for(self, rows: int):
+        """(weight, eps) if, in a step of `rows` rows, whatever writes the residual before this norm
+        may prepare its rows instead (see `OwedRows`: the consumer's product then pays the scale and
+        no norm kernel runs); None if this norm wants to run its own kernel.  The limits are those of
+        the products that pay: bfloat16, few rows, rows of 16-byte multiples."""
+        if self.dtype != torch.bfloat16 or not 0 < rows <= K.FOLD_MAX_ROWS or self.spec.size % 8:
+            return None
         return self.weight, self.spec.eps
+
+    def decode_fusable(self, rows: int, block_size: int) -> bool:
+        return self.folded_for(rows) is not None  # then `forward` hands prepared rows on and launches nothing
 
     def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None):
         """Add the pending branch output into the residual and return the normalised

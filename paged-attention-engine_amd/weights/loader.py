@@ -50,6 +50,10 @@ def _open_shards(model_dir: str) -> Dict[str, SafetensorsFile]:
         absent = []  # names the index sends to a shard that does not hold them
         for name, shard in weight_map.items():
             if shard not in files:
+                # the index is as little to be trusted as the checkpoint: a shard is a file of this folder
+                if not isinstance(shard, str) or not shard or os.path.basename(shard) != shard or shard in (".", ".."):
+                    raise WeightsError(f"{index_path}: the entry '{name}' names the shard {shard!r}, "
+                                       "which is not a plain file name inside the model folder")
                 shard_path = os.path.join(model_dir, shard)
                 if not os.path.exists(shard_path):
                     raise WeightsError(f"{index_path} names the shard {shard}, which is not in the folder")

@@ -31,10 +31,6 @@ def _tensor_seed(seed: int, name: str) -> int:
     return (int(seed) * 1000003 + zlib.crc32(name.encode("utf-8"))) & 0x7FFFFFFFFFFFFFFF
 
 
-def is_norm_weight(name: str) -> bool:
-    return name.endswith("norm.weight") or name.endswith("layernorm.weight")
-
-
 def std_of(name: str, std) -> float:
     """`std` is one number for every tensor, or a mapping from name endings to numbers with the
     fallback under "" (so that, say, query and key projections can be drawn wider than the rest
@@ -50,10 +46,15 @@ def std_of(name: str, std) -> float:
 def random_tensor(name: str, shape: Tuple[int, ...], seed: int, std=0.02,
                   norm_std: float = 0.0, device: str = "cpu",
                   dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """`shape` is what the part declared: a plain tuple is drawn about zero with `std`; a shape with
+    a `centre` (a tensor that scales activations, see `parts.ScaleShape`) about that centre with
+    `norm_std`.  Nothing is read from the tensor's name but its seed and, if `std` is a mapping, its std."""
     gen = torch.Generator(device=device).manual_seed(_tensor_seed(seed, name))
     std = std_of(name, std)
-    if is_norm_weight(name):
-        t = torch.ones(shape, device=device)
+    centre = float(getattr(shape, "centre", 0.0))
+    shape = tuple(shape)
+    if centre:
+        t = torch.full(shape, centre, device=device)
         if norm_std:
             t += norm_std * torch.randn(shape, generator=gen, device=device)
     else:
@@ -65,7 +66,7 @@ def random_tensor(name: str, shape: Tuple[int, ...], seed: int, std=0.02,
 def random_weights(expected: Mapping[str, Tuple[int, ...]], seed: int, std=0.02,
                    norm_std: float = 0.0, device: str = "cpu",
                    dtype: torch.dtype = torch.bfloat16) -> Dict[str, torch.Tensor]:
-    return {name: random_tensor(name, tuple(shape), seed, std, norm_std, device, dtype)
+    return {name: random_tensor(name, shape, seed, std, norm_std, device, dtype)
             for name, shape in expected.items()}
 
 
@@ -76,7 +77,7 @@ class RandomWeights(Mapping):
 
     def __init__(self, expected: Mapping[str, Tuple[int, ...]], seed: int, std=0.02,
                  norm_std: float = 0.0, device: str = "cuda:0", dtype: torch.dtype = torch.bfloat16) -> None:
-        self.shapes = {name: tuple(shape) for name, shape in expected.items()}
+        self.shapes = dict(expected)  # as declared: a shape may say how its tensor is drawn
         self.seed, self.std, self.norm_std, self.device, self.dtype = seed, std, norm_std, device, dtype
 
     def __getitem__(self, name: str) -> torch.Tensor:

@@ -41,7 +41,7 @@ TINY_D = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=2, hidden_si
 # heads per key/value head, a window on the second layer.  Query and key projections are drawn
 # six times wider than the rest, so that scores spread over several units and attention is peaked:
 # a missing rotation or a flat softmax then moves the logits far beyond the bfloat16 tolerance
-# (tests/test_gpu_sensitivity.py shows by how much).
+# (`test_the_peaked_model_shows_mistakes...` in tests/test_plain.py shows by how much).
 TINY_E = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=2, hidden_size=192,
               num_attention_heads=12, num_key_value_heads=2, head_dim=64, intermediate_size=328,
               vocab_size=1500, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,

@@ -70,6 +70,28 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return weight.to(in_dtype) * xw.to(in_dtype)
 
 
+# The precision in which rotation angles are formed in `self_attention`: None = the working precision
+# of the call.  The reference forms them in float32 whatever the activations' type (engine/model.py:
+# 132-152: inv_freq and positions * inv_freq "built in float32 then cast"); at position 2,000 a float32
+# angle is 1e-4 radians away from the float64 one, which the scores of a peaked model turn into logit
+# differences several times the float32 comparison bound, so comparisons of a float32 engine at long
+# positions set this to torch.float32 (`angles_in`): everything else stays in the working precision.
+ANGLE_DTYPE = None
+
+
+class angles_in:
+    def __init__(self, dtype):
+        self.dtype = dtype
+
+    def __enter__(self):
+        global ANGLE_DTYPE
+        self.saved, ANGLE_DTYPE = ANGLE_DTYPE, self.dtype
+
+    def __exit__(self, *exc):
+        global ANGLE_DTYPE
+        ANGLE_DTYPE = self.saved
+
+
 def rope_inv_freq(head_dim: int, theta: float, work: torch.dtype = torch.float32, device=None) -> torch.Tensor:
     """engine/model.py:132-135 -- 1 / theta ** (arange(0, hd, 2) / hd)."""
     exponent = torch.arange(0, head_dim, 2, dtype=torch.int64, device=device).to(work)
@@ -81,6 +103,8 @@ def rope_cos_sin(inv_freq: torch.Tensor, positions: torch.Tensor, dtype: torch.d
     cos and sin taken in the working precision, then cast to `dtype`."""
     freqs = positions.to(inv_freq.dtype)[:, None] * inv_freq[None, :]
     emb = torch.cat((freqs, freqs), dim=-1)
+    if dtype == torch.float64:  # cosine and sine of the angle as formed, not rounded to its precision
+        emb = emb.double()
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
@@ -167,7 +191,8 @@ def self_attention(w: dict, prefix: str, cfg: dict, x: torch.Tensor, positions: 
     k = split_heads(linear(x, w[p + "k_proj.weight"], w[p + "k_proj.bias"]), nkv, hd)
     v = split_heads(linear(x, w[p + "v_proj.weight"], w[p + "v_proj.bias"]), nkv, hd)
     work = torch.float64 if x.dtype == torch.float64 else torch.float32
-    cos, sin = rope_cos_sin(rope_inv_freq(hd, rope_theta_of(cfg), work, x.device), positions, x.dtype)
+    angle = ANGLE_DTYPE or work
+    cos, sin = rope_cos_sin(rope_inv_freq(hd, rope_theta_of(cfg), angle, x.device), positions, x.dtype)
     q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
     out = attention(q, k, v, hd ** -0.5, window)
     return linear(merge_heads(out), w[p + "o_proj.weight"])

@@ -208,13 +208,21 @@ def test_the_pool_is_sized_once_in_pages_or_bytes_or_a_share_of_free_memory():
 def test_random_weights_are_drawn_at_the_lookup_and_repeat():
     from paged_attention_engine_amd.weights import RandomWeights
 
-    shapes = {"a.q_proj.weight": (6, 4), "a.input_layernorm.weight": (4,), "b.weight": (3, 3)}
+    from paged_attention_engine_amd.parts import ScaleShape
+
+    # how a tensor is drawn is said where it is declared, not read off its name: the scale vector is
+    # called `ln.scale` here, and a matrix whose name ends like a norm's weight stays a matrix
+    shapes = {"a.q_proj.weight": (6, 4), "a.ln.scale": ScaleShape((4,)), "b.weight": (3, 3),
+              "c.input_layernorm.weight": (64, 8)}
+    assert shapes["a.ln.scale"] == (4,)
     drawn = RandomWeights(shapes, seed=5, std={"": 0.02, "q_proj.weight": 0.5}, norm_std=0.1, device="cpu")
-    assert sorted(drawn) == sorted(shapes) and len(drawn) == 3
+    assert sorted(drawn) == sorted(shapes) and len(drawn) == 4
     first, again = drawn["a.q_proj.weight"], drawn["a.q_proj.weight"]
     assert first is not again and torch.equal(first, again) and first.dtype == torch.bfloat16
     assert float(first.float().std()) > 0.2 > float(drawn["b.weight"].float().std())  # the wider ending applies
-    assert float((drawn["a.input_layernorm.weight"].float() - 1).abs().max()) < 0.5
+    assert float((drawn["a.ln.scale"].float() - 1).abs().max()) < 0.5
+    assert float((RandomWeights(shapes, seed=5, device="cpu")["a.ln.scale"].float() - 1).abs().max()) == 0.0
+    assert float(drawn["c.input_layernorm.weight"].float().abs().max()) < 0.2  # about zero: it was declared a matrix
     assert not torch.equal(first, RandomWeights(shapes, seed=6, device="cpu")["a.q_proj.weight"])
     with pytest.raises(KeyError):
         drawn["c"]
@@ -238,6 +246,21 @@ def test_an_index_that_names_what_a_shard_lacks_is_a_weights_error(tmp_path):
         load_weights(str(tmp_path), {"a": (2, 2), "b": (2, 2)})
 
 
+def test_a_shard_index_cannot_reach_outside_the_model_folder(tmp_path):
+    import json
+
+    from paged_attention_engine_amd.weights import load_weights, save_file
+
+    outside = tmp_path / "elsewhere.safetensors"
+    save_file({"a": torch.zeros(2, 2)}, str(outside))
+    folder = tmp_path / "model"
+    folder.mkdir()
+    for shard in ("../elsewhere.safetensors", str(outside), "sub/x.safetensors", "..", ""):
+        (folder / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"a": shard}}))
+        with pytest.raises(pae.WeightsError, match="plain file name"):
+            load_weights(str(folder), {"a": (2, 2)})
+
+
 def test_loaded_weights_are_views_of_the_file(tmp_path):
     from paged_attention_engine_amd.weights import load_weights, save_file
 
@@ -248,3 +271,31 @@ def test_loaded_weights_are_views_of_the_file(tmp_path):
     assert torch.equal(weights["a"], torch.arange(6, dtype=torch.float32).view(2, 3))
     assert weights["h"].dtype == torch.float32  # half precision is widened, nothing else is copied
     assert weights.get("zzz") is None
+
+
+def test_the_default_precision_is_the_configs_own():
+    from paged_attention_engine_amd.engine.model import default_dtype
+
+    cfg = dict(helpers.TINY_A)
+    assert default_dtype(pae.read_config_dict(cfg)) == "bfloat16"
+    assert default_dtype(pae.read_config_dict(dict(cfg, torch_dtype="float32"))) == "float32"
+    assert default_dtype(pae.read_config_dict(dict(cfg, torch_dtype="torch.float32"))) == "float32"
+    assert default_dtype(pae.read_config_dict(dict(cfg, torch_dtype="float16"))) == "bfloat16"  # served in bfloat16
+    assert pae.read_config_dict(dict(cfg, torch_dtype="float32")).to_json_dict()["torch_dtype"] == "float32"
+
+
+def test_state_slots_bound_live_sequences_only_where_someone_said_so():
+    from paged_attention_engine_amd.config.engine_config import EngineConfig
+
+    assert EngineConfig(num_state_slots=5, max_num_seqs=9).state_slots_for(100, True) == 5
+    assert EngineConfig(max_num_seqs=9).state_slots_for(100, False) == 9
+    # nobody said: a model without per-request state gets a slot per page, which never binds
+    assert EngineConfig().state_slots_for(100, False) == 100
+    with pytest.raises(ValueError, match="max_num_seqs or num_state_slots"):
+        EngineConfig().state_slots_for(100, True)
+
+
+def test_a_plan_names_the_tensors_a_checkpoint_may_hold_unused():
+    tied = pae.read_config_dict(dict(helpers.TINY_A, tie_word_embeddings=True)).plan()
+    untied = pae.read_config_dict(dict(helpers.TINY_A, tie_word_embeddings=False)).plan()
+    assert tied.optional_names == ("lm_head.weight",) and untied.optional_names == ()

@@ -83,10 +83,37 @@ def test_command_line_generates_the_same_tokens(tmp_path):
     assert sorted(os.listdir(tmp_path / "saved")) == ["config.json", "model.safetensors"]
 
 
+def test_command_line_draws_random_weights_on_the_device_and_sizes_the_pool_by_bytes(tmp_path):
+    """`--random-config` without `--save-model` draws the weights on the GPU and writes nothing; the
+    pool is sized as a share of the free memory or by a byte budget, which changes no token; without
+    `--dtype` the precision is the config's `torch_dtype`."""
+    cfg_path = tmp_path / "cfg.json"
+    cfg_path.write_text(json.dumps(dict(helpers.TINY_A, torch_dtype="float32")))
+
+    def run(*extra):
+        out = subprocess.run([sys.executable, "-m", "paged_attention_engine_amd", "--random-config", str(cfg_path),
+                              "--seed", "3", "--prompt-ids", "5,17,3,99", "--prompt-ids", "8 9 10",
+                              "--max-new-tokens", "7", "--dump-logits", str(tmp_path / "logits.pt"), *extra],
+                             cwd=ROOT, capture_output=True, text=True)
+        assert out.returncode == 0, out.stderr[-2000:]
+        lines = [json.loads(line) for line in out.stdout.splitlines() if line.startswith("{")]
+        return [line["token_ids"] for line in lines], torch.load(tmp_path / "logits.pt", weights_only=True)
+
+    by_share, logits = run("--fill-hbm", "0.05")
+    assert [len(t) for t in by_share] == [7, 7]
+    assert logits["r0"].dtype == torch.float32 and logits["r0"].shape == (7, helpers.TINY_A["vocab_size"])
+    by_bytes, logits_again = run("--kv-bytes", str(1 << 22))
+    assert by_bytes == by_share and torch.equal(logits_again["r0"], logits["r0"])  # float32: bit for bit
+    in_bf16, _ = run("--kv-bytes", str(1 << 22), "--dtype", "bfloat16")
+    assert [len(t) for t in in_bf16] == [7, 7]
+    assert sorted(os.listdir(tmp_path)) == ["cfg.json", "logits.pt"]  # no model folder was written
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(tmp_path, dtype):
-    """400 decoded tokens: pages fill one after the other, the windowed group of model D gives
-    pages back on the way, and HIP graphs are re-recorded as the block tables widen."""
+    """400 decoded tokens: pages fill one after the other and the windowed group of model D gives
+    pages back on the way.  (The tables stay below 64 pages here; recorded steps whose tables grow
+    past that are covered in tests/test_gpu_long_context.py.)"""
     for name in ("B", "D"):
         folder = helpers.make_model_folder(tmp_path, name)
         cfg, weights = helpers.read_folder_plain(folder)

@@ -226,13 +226,18 @@ class ToyConfig:
     def plan(self):
         c = self.cfg
         H, hd = c["hidden_size"], c["head_dim"]
-        norm = NormSpec(size=H, eps=c["eps"])
+        # names of this architecture's own: norms are `ln1.scale` / `ln2.scale` / `final_ln.scale`, the
+        # attention's projections `wq` .. `wo` (the built-in parts take their names from the specs)
+        norm = NormSpec(size=H, eps=c["eps"], weight_name="scale")
         attn = MixerSpec(hidden_size=H, num_heads=c["heads"], num_kv_heads=c["kv_heads"], head_dim=hd,
-                         scale=hd ** -0.5, qkv_bias=False, position=PositionSpec(kind="toy_shift"))
+                         scale=hd ** -0.5, qkv_bias=False, position=PositionSpec(kind="toy_shift"),
+                         q_name="wq", k_name="wk", v_name="wv", o_name="wo")
         ffn = FeedForwardSpec(hidden_size=H, intermediate_size=c["inter"])
-        layers = (LayerSpec("layers.0.", attn, ffn, norm, norm), LayerSpec("layers.1.", DecaySpec(hidden_size=H, decay=c["decay"]), ffn, norm, norm))
+        names = dict(mixer_norm_prefix="ln1.", feed_forward_norm_prefix="ln2.")
+        layers = (LayerSpec("layers.0.", attn, ffn, norm, norm, **names),
+                  LayerSpec("layers.1.", DecaySpec(hidden_size=H, decay=c["decay"]), ffn, norm, norm, **names))
         schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(0, cache_from=0), ScheduleEntry(1))
-        return ModelPlan("ToyForCausalLM", H, c["vocab"], layers, schedule, norm, "embed.weight", "head.weight", "final_norm.",
+        return ModelPlan("ToyForCausalLM", H, c["vocab"], layers, schedule, norm, "embed.weight", "head.weight", "final_ln.",
                          embedding_scale=c["embedding_scale"], logit_scale=c["logit_scale"], logit_softcap=c["logit_softcap"])
 
 
@@ -250,16 +255,16 @@ def toy_plain_logits(w, c, ids):
 
     def attention(prefix, h, borrowed=None):
         nh, nkv, hd = c["heads"], c["kv_heads"], c["head_dim"]
-        q = plain.split_heads(plain.linear(h, w[prefix + "q_proj.weight"].double()), nh, hd).clone()
+        q = plain.split_heads(plain.linear(h, w[prefix + "wq.weight"].double()), nh, hd).clone()
         q[:, :, 0] += pos / 100.0
         if borrowed is None:
-            k = plain.split_heads(plain.linear(h, w[prefix + "k_proj.weight"].double()), nkv, hd).clone()
-            v = plain.split_heads(plain.linear(h, w[prefix + "v_proj.weight"].double()), nkv, hd)
+            k = plain.split_heads(plain.linear(h, w[prefix + "wk.weight"].double()), nkv, hd).clone()
+            v = plain.split_heads(plain.linear(h, w[prefix + "wv.weight"].double()), nkv, hd)
             k[:, :, 0] += pos / 100.0
         else:
             k, v = borrowed
         out = plain.attention(q, k, v, hd ** -0.5)
-        return plain.linear(plain.merge_heads(out), w[prefix + "o_proj.weight"].double()), (k, v)
+        return plain.linear(plain.merge_heads(out), w[prefix + "wo.weight"].double()), (k, v)
 
     def decay(prefix, h):
         u = h @ w[prefix + "in.weight"].double().t()
@@ -271,7 +276,7 @@ def toy_plain_logits(w, c, ids):
 
     for stop, (layer, borrow) in enumerate(((0, False), (1, False), (0, False), (0, True), (1, False))):
         p = f"layers.{layer}."
-        h = plain.rms_norm(x, w[p + "input_layernorm.weight"].double(), c["eps"])
+        h = plain.rms_norm(x, w[p + "ln1.scale"].double(), c["eps"])
         if layer == 0:
             y, kv = attention(p + "self_attn.", h, kv_of_stop0 if borrow else None)
             if stop == 0:
@@ -279,9 +284,9 @@ def toy_plain_logits(w, c, ids):
         else:
             y = decay(p + "self_attn.", h)
         x = x + y
-        h = plain.rms_norm(x, w[p + "post_attention_layernorm.weight"].double(), c["eps"])
+        h = plain.rms_norm(x, w[p + "ln2.scale"].double(), c["eps"])
         x = x + plain.swiglu_mlp({k: v.double() for k, v in w.items()}, p, h)
-    logits = c["logit_scale"] * plain.linear(plain.rms_norm(x, w["final_norm.weight"].double(), c["eps"]),
+    logits = c["logit_scale"] * plain.linear(plain.rms_norm(x, w["final_ln.scale"].double(), c["eps"]),
                                              w["head.weight"].double())
     return c["logit_softcap"] * torch.tanh(logits / c["logit_softcap"])
 
@@ -322,9 +327,15 @@ def test_toy_routed_feed_forward_is_registered_and_built(dtype):
 def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
     assert "ToyForCausalLM" in pae.known_architectures()
     config = pae.read_config_dict(TOY)
-    folder = pae.write_model_folder(config, 5, str(tmp_path / "toy"), std=0.08)
+    folder = pae.write_model_folder(config, 5, str(tmp_path / "toy"), std=0.08, norm_std=0.1)
     model = pae.load_model(folder, dtype)
     assert not model.graph_safe  # the toy parts run host loops: steps are launched eagerly
+    # random mode draws a tensor as the part that declares it says, whatever it is called: this
+    # architecture's norm weights are `...ln1.scale`, and they come out about one
+    drawn = pae.random_model(config, 5, dtype, std=0.08, norm_std=0.1)
+    for norm_part in (drawn.blocks[0].mixer_norm, drawn.blocks[1].feed_forward_norm, drawn.final_norm):
+        assert 0.05 < float((norm_part.weight.float() - 1).abs().max()) < 0.6
+    assert {"layers.0.ln1.scale", "layers.1.ln2.scale", "final_ln.scale", "layers.0.self_attn.wq.weight"} <= set(drawn.expected_tensors())
     paged, states = model.cache_specs()
     assert [p is not None for p in paged] == [True, False, True, False, False]  # stop 3 borrows stop 0's cache
     assert [s is not None for s in states] == [False, True, False, False, True]

@@ -3,8 +3,9 @@
 `pae_sample_static` keeps its chunk results in a buffer inside the library's image on the GPU.
 Two calls in a row, the second with fewer rows and a shorter vocabulary (so that it finds the first
 call's leftovers in the buffer), must give exactly what `pae_sample` gives with a workspace of the
-caller's; sizes beyond the buffer are refused with a message; and no device memory is taken from
-the driver by the calls.
+caller's; sizes beyond the buffer are refused with a message; no device memory is taken from
+the driver by the calls (by the driver's own count of free memory); and the call can be recorded
+into a graph once the buffer's address is known.
 """
 
 import ctypes
@@ -57,6 +58,7 @@ def test_sampling_without_a_workspace_matches_sampling_with_one():
     want_second = _reference(*second)
     want_greedy = _reference(second[0], None, None)
     torch.cuda.synchronize()
+    # what the driver itself says is free: torch's own counters cannot see a hipMalloc inside the library
     held = torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0]
 
     code, got_first = _static(lib, *first)
@@ -72,8 +74,35 @@ def test_sampling_without_a_workspace_matches_sampling_with_one():
     assert int(got_first.min()) >= 0 and int(got_first.max()) < 151_937
     # greedy rows are the first maximum
     assert torch.equal(got_greedy.long(), second[0].argmax(dim=1))
-    # the tokens of this test's own outputs aside, nothing was taken from the driver
+    # nothing was taken from the driver, neither by torch (the outputs' few bytes come out of blocks it
+    # already holds) nor behind its back by the library
     assert torch.cuda.memory_reserved() == held[0]
+    assert torch.cuda.mem_get_info()[0] == held[1]
+
+
+def test_the_call_can_be_recorded_into_a_graph_after_a_first_call_outside():
+    """The buffer's address is looked up at the first call on a device, which must not fall inside a
+    capture; after it, the call records like any kernel launch.  Every replay is checked against the
+    eager result, with eager work and synchronisation between the replays."""
+    device = torch.device("cuda:0")
+    lib = K.library()
+    assert lib.pae_sample_static_prepare() == 0, lib.pae_last_error()
+    logits, temperature, uniform = _case(9, 50_021, 11, device)
+    tokens = torch.full((9,), -7, dtype=torch.int32, device=device)
+    K.sample_static(tokens, logits, temperature, uniform)  # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        K.sample_static(tokens, logits, temperature, uniform)
+    for seed in (12, 13, 14):
+        fresh = _case(9, 50_021, seed, device)
+        want = _reference(*fresh)
+        for dst, src in zip((logits, temperature, uniform), fresh):
+            dst.copy_(src)
+        tokens.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(tokens, want), seed
 
 
 def test_sizes_beyond_the_buffer_are_refused():
