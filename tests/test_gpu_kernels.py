@@ -165,6 +165,90 @@ def test_a_norm_folded_into_the_products_around_it(M, N, K_, ranges):
     assert (plain_rows.double().cpu() - normed).abs().max() <= 2.0 ** -6 * float(normed.abs().max())
 
 
+@pytest.mark.parametrize("N,K_", [(1536, 1536), (1536, 8960), (2048, 1536), (17920, 1536), (3584, 18944), (4608, 3584),
+                                  (200, 1032), (1000, 264)])
+def test_a_rows_sums_do_not_depend_on_the_batch_up_to_16_rows(N, K_):
+    """Up to 16 rows every product takes its k ranges from its sizes alone and adds them in one order,
+    whichever kernel runs them (one workgroup of sixteen wavefronts for four ranges side by side, or
+    a workgroup per range and a ticket): a row alone, among 8 rows and among 16 gives the same bits,
+    through the plain, the gated and the residual epilogue, with and without a row scale."""
+    torch.manual_seed(N + K_)
+    a = (torch.randn(16, K_) * 0.5).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K_) * 0.1).to(torch.bfloat16).to(DEV)
+    stats_in = (torch.rand(16, K().stat_tiles(K_)) + 0.5).to(DEV)
+    residual = (torch.randn(16, N) * 2.0).to(DEV)
+    w_norm = (1 + 0.2 * torch.randn(N)).to(torch.bfloat16).to(DEV)
+
+    def run(rows, epilogue, scaled):
+        M = len(rows)
+        x = a[rows].contiguous()
+        scale = (stats_in[rows].contiguous(), 1e-6) if scaled else None
+        if epilogue == K().EPI_RESIDUAL:
+            out = residual[rows].clone()
+            nxt = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            stats = torch.empty(M, K().stat_tiles(N), dtype=torch.float32, device=DEV)
+            K().gemm_skinny(out, x, w, None, epilogue, K().residual_splits(N, K_, M), scale, (nxt, w_norm, stats))
+            return out, nxt, stats
+        cols = N // 2 if epilogue == K().EPI_SWIGLU else N
+        out = torch.empty(M, cols, dtype=torch.bfloat16, device=DEV)
+        K().gemm_skinny(out, x, w, None, epilogue, K().whole_sum_splits(N, K_, M), scale)
+        return (out,)
+
+    epilogues = [K().EPI_BF16, K().EPI_RESIDUAL] + ([K().EPI_SWIGLU] if N % 16 == 0 else [])
+    for epilogue in epilogues:
+        for scaled in (False, True):
+            alone = run([5], epilogue, scaled)
+            eight = run(list(range(8)), epilogue, scaled)
+            twelve = run(list(range(2, 14)), epilogue, scaled)
+            sixteen = run(list(range(16)), epilogue, scaled)
+            for t_alone, t8, t12, t16 in zip(alone, eight, twelve, sixteen):
+                assert torch.equal(t_alone[0], t8[5]) and torch.equal(t_alone[0], t12[3]) and torch.equal(t_alone[0], t16[5])
+    # four ranges side by side in one workgroup are the four ranges of separate workgroups, bit for bit
+    if K().residual_splits(N, K_, 8) == 4:
+        side_by_side = run(list(range(8)), K().EPI_RESIDUAL, True)
+        program = K().DecodeProgram(DEV, 2)  # a decode program's product phase always goes by tickets
+        out = residual[:8].clone()
+        nxt = torch.empty(8, N, dtype=torch.bfloat16, device=DEV)
+        stats = torch.empty(8, K().stat_tiles(N), dtype=torch.float32, device=DEV)
+        with K().recording(program):
+            K().gemm_skinny(out, a[:8].contiguous(), w, None, K().EPI_RESIDUAL, 4, (stats_in[:8].contiguous(), 1e-6),
+                            (nxt, w_norm, stats))
+        program.launch()
+        torch.cuda.synchronize()
+        program.check()
+        for got, want in zip((out, nxt, stats), side_by_side):
+            assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("M,N,K_,ranges", [(8, 1536, 8960, 1), (8, 1536, 1536, 4), (12, 18944, 3584, 1), (16, 3584, 18944, 4),
+                                            (7, 1000, 1032, 3), (16, 72, 2048, 4), (3, 200, 8, 1)])
+def test_the_residual_epilogue_on_every_branch_of_its_launcher(M, N, K_, ranges):
+    """One range, four ranges side by side in a workgroup of sixteen wavefronts, ticketed ranges, a
+    width that is no multiple of 16: the residual, the next rows and the sums of squares against a
+    float64 computation, tightly."""
+    torch.manual_seed(M + N + K_)
+    a = (torch.randn(M, K_) * 0.5).to(torch.bfloat16)
+    w = (torch.randn(N, K_) * 0.1).to(torch.bfloat16)
+    residual = torch.randn(M, N) * 2.0
+    w_norm = (1 + 0.2 * torch.randn(N)).to(torch.bfloat16)
+    want = residual.double() + a.double() @ w.double().t()
+    res_d = residual.to(DEV)
+    nxt = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    stats = torch.full((M, K().stat_tiles(N)), float("nan"), dtype=torch.float32, device=DEV)
+    K().gemm_skinny(res_d, a.to(DEV), w.to(DEV), None, K().EPI_RESIDUAL, ranges, following=(nxt, w_norm.to(DEV), stats))
+    top = float(want.abs().max())
+    assert (res_d.double().cpu() - want).abs().max() <= 4e-6 * top + 1e-6
+    rows = (res_d.cpu() * w_norm.float()).to(torch.bfloat16)
+    assert torch.equal(nxt.cpu(), rows)  # the rounding of exactly the residual that was written
+    assert torch.isfinite(stats).all()
+    assert torch.allclose(stats.double().cpu().sum(1), res_d.double().cpu().pow(2).sum(1), rtol=2e-6)
+    # every share is its own 16 columns' sum of squares
+    padded = torch.zeros(M, K().stat_tiles(N) * 16, dtype=torch.float64)
+    padded[:, :N] = res_d.double().cpu().pow(2)
+    assert torch.allclose(stats.double().cpu(), padded.view(M, -1, 16).sum(-1), rtol=2e-6, atol=1e-12)
+    K().check_tickets_zero(DEV)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_embedding_rows(dtype):
     torch.manual_seed(3)

@@ -125,3 +125,41 @@ def test_a_part_that_is_not_recordable_is_refused_while_recording():
             K.swiglu(torch.empty(4, 32, dtype=torch.bfloat16, device="cuda:0"), x)
     assert program.count == 0
     K.swiglu(torch.empty(4, 32, dtype=torch.bfloat16, device="cuda:0"), x)  # and works again afterwards
+
+
+@pytest.mark.parametrize("programs", [False, True])
+def test_a_sequences_decoded_logits_do_not_depend_on_the_batch_up_to_16_rows(tmp_path, programs):
+    """Decode steps of up to 16 sequences add every product's k in one order and split the attention
+    at fixed places: a sequence decoded alone, beside 7 others and beside 15 others gives the same
+    logits bit for bit (prompts run alone in all three, so the caches start equal), at the real layer
+    widths, with the kernels launched one by one or as a program."""
+    model = pae.random_model(WIDE, seed=5, dtype="bfloat16")
+    lengths = (200, 9, 100, 250, 31, 64, 65, 1, 300, 4, 127, 128, 129, 77, 16, 17)
+    prompts = [tokens(WIDE["vocab_size"], n, 21 + n) for n in lengths]
+    steps = 5
+    feed = [[tokens(WIDE["vocab_size"], 1, 1000 * step + s)[0] for s in range(16)] for step in range(steps)]
+
+    def decode(which):
+        pages = sum(-(-(len(prompts[s]) + steps) // 16) + 1 for s in which) + 2
+        cache = model.new_cache(16, pages, len(which))
+        runner = pae.StepRunner(model, cache, use_graphs=False, use_programs=programs)
+        for s in which:
+            assert cache.create_sequence(s)
+            cache.reserve(s, len(prompts[s]))
+            runner.run([pae.StepEntry(s, tuple(prompts[s]), ())])
+        out = []
+        for step in range(steps):
+            entries = []
+            for s in which:
+                cache.reserve(s, 1)
+                entries.append(pae.StepEntry(s, (feed[step][s],), (0,)))
+            out.append(runner.run(entries).clone())
+        torch.cuda.synchronize()
+        runner.check_programs()
+        return torch.stack(out)  # [step, sequence, vocab]
+
+    alone = decode([0])
+    eight = decode(list(range(8)))
+    sixteen = decode(list(range(16)))
+    assert torch.equal(alone[:, 0], eight[:, 0]) and torch.equal(alone[:, 0], sixteen[:, 0])
+    assert torch.equal(eight, sixteen[:, :8])
