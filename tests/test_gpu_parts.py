@@ -74,6 +74,55 @@ def test_norm_part(dtype):
     assert stream.pending is not None and (rows.double().cpu() - want2).abs().max() <= TOL[dtype] * 4
 
 
+def test_norm_part_and_rows_that_a_product_prepared():
+    """A branch's last product may have added itself into the residual and prepared rows for a norm.
+    The norm they were prepared for hands them on as they are (no kernel); another norm, or the same
+    norm asked for some rows only, normalises the (complete) residual itself."""
+    torch.manual_seed(4)
+    width, eps = 200, 3e-6
+    spec = NormSpec(size=width, eps=eps)
+    mine, other = (P.build_part(P.NORMS, "norm", spec, torch.bfloat16, DEV) for _ in range(2))
+    w_mine, w_other = (1 + 0.1 * torch.randn(width)).bfloat16(), (1 + 0.3 * torch.randn(width)).bfloat16()
+    mine.bind("a.", {"a.weight": w_mine})
+    other.bind("b.", {"b.weight": w_other})
+    assert mine.folded_for(3) is not None and mine.folded_for(17) is None and mine.folded_for(0) is None
+    assert P.build_part(P.NORMS, "norm", spec, torch.float32, DEV).folded_for(3) is None  # float32 runs its kernel
+    res = torch.randn(3, width)
+    rows = (res * w_mine.float()).bfloat16()
+    stats = torch.zeros(3, K_stat_tiles(width))
+    padded = torch.zeros(3, K_stat_tiles(width) * 16)
+    padded[:, :width] = res.pow(2)
+    stats = padded.view(3, -1, 16).sum(-1)
+
+    def stream_with_owed(to):
+        stream = P.ResidualStream(res.to(DEV))
+        stream.owed, stream.owed_to = P.OwedRows(rows.to(DEV), stats.to(DEV), eps), to
+        return stream
+
+    stream = stream_with_owed(mine)
+    handed = stream.owed
+    got = mine.forward(stream)
+    assert got is handed and stream.owed is None  # handed on as they are: no kernel ran
+    settled = P.plain_rows(got)
+    want = plain.rms_norm(res.double(), w_mine.double(), eps)
+    assert (settled.double().cpu() - want).abs().max() <= TOL["bfloat16"] * 4
+    # prepared for another norm: this one normalises the residual with its own weight
+    stream = stream_with_owed(other)
+    got = mine.forward(stream)
+    assert torch.is_tensor(got) and stream.owed is None
+    assert (got.double().cpu() - want).abs().max() <= TOL["bfloat16"] * 4
+    # some rows only: the stream keeps what it owes, the rows come from the residual
+    stream = stream_with_owed(mine)
+    got = mine.forward(stream, torch.tensor([2, 0], dtype=torch.int32, device=DEV))
+    assert torch.is_tensor(got) and stream.owed is not None and stream.owed_to is mine
+    assert (got.double().cpu() - want[[2, 0]]).abs().max() <= TOL["bfloat16"] * 4
+
+
+def K_stat_tiles(width):
+    from paged_attention_engine_amd.kernels import lib
+    return lib.stat_tiles(width)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("hidden,inter", [(96, 208), (72, 200)])  # the second is not a multiple of 16
 def test_feed_forward_part(dtype, hidden, inter):
