@@ -18,9 +18,12 @@
 //
 // What one workgroup writes and another reads after the barrier is written through to the memory
 // side with device-scope stores (the dies' L2s are not coherent with one another, see
-// skinny_device.h), acknowledged before the workgroup arrives at the barrier, and every wavefront
-// invalidates its caches after the barrier before it reads.  Every wait is bounded: a workgroup
-// that has polled `spin_limit` times gives up, leaves an error code for the host and for the other
+// skinny_device.h), acknowledged before the workgroup arrives at the barrier, and read with
+// device-scope loads, which are served past the reader's own L2 (dropping the L2's contents after
+// every barrier instead costs 1.7 us a barrier).  So that those loads stay few, a product's
+// activations are read once per workgroup, into LDS.  Weights, tables and the cache's older pages,
+// which nobody writes during the step, are read plainly.  Every wait is bounded: a workgroup that
+// has polled `spin_limit` times gives up, leaves an error code for the host and for the other
 // workgroups, and the kernel ends.
 #include "common.h"
 #include "api.h"
@@ -91,7 +94,8 @@ __device__ __forceinline__ unsigned barrier_epoch_at_start(const ProgBarrier* ba
   return __hip_atomic_load(&bar->die[die][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) / barrier_members(die);
 }
 
-// True when every workgroup has arrived and the caches are clean; false when the program is dead
+// True when every workgroup has arrived (what they wrote through is then in memory; the reader's caches
+// may still hold older copies, which is why it reads such data with device-scope loads); false when the program is dead
 // (this workgroup or another gave up), in which case the kernel must end.  `epoch` lives in thread 0.
 __device__ __forceinline__ bool grid_barrier(ProgBarrier* bar, unsigned& epoch, int* s_dead, int spin_limit, int phase) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's written-through stores have arrived
@@ -118,55 +122,61 @@ __device__ __forceinline__ bool grid_barrier(ProgBarrier* bar, unsigned& epoch, 
       __hip_atomic_store(&bar->error[0], (unsigned)(phase + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       *s_dead = 1;
     }
-    // Nothing read below may come from a stale cache line: the compute unit's vector cache and the
-    // die's L2 drop what they hold of memory that other dies may have written.  Once a workgroup is
-    // enough (its wavefronts share the caches); every wavefront doing it costs 30 us a barrier.
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   }
   __syncthreads();
   return *s_dead == 0;
 }
 
 // ---------------------------------------------------------------------------------------- product
-// Item i of a product phase is tile i % tiles of 16 weight rows over k range i / tiles; quad q of
-// workgroup b takes the items base + q * gridDim.x + b of every round.  The quad's four wavefronts
-// take the 32-wide k steps of the range in turn and their sums are added in wavefront order through
-// LDS (two buffers that take turns, so that a round needs one workgroup barrier).
+// A product phase is cut into items of 16 weight rows (a tile) by one k range.  A workgroup serves one
+// k range (workgroup b the range b % splits; with fewer workgroups than ranges, several in turn): it
+// reads the activations of that range once, with device-scope loads, into LDS, in the order in which the
+// matrix instruction wants its B operand, and its quads then take the range's tiles in turn, streaming
+// only weights.  A quad's four wavefronts take the 32-wide k steps of the range in turn and their sums
+// are added in wavefront order through LDS, exactly as gemm_skinny_kernel<1, 1, EPI, 4> adds them.
 //
-// A quad asks for the first fragments of its coming item while the current one finishes: the weights
-// and activations of the next round's item, or, at the end of the phase, the weights of its first item
-// of the next phase (weights do not depend on what the barrier waits for; activations do, and are
-// asked for behind it).  `Ahead` carries them from item to item and from phase to phase.
-#define PROG_U 4  // k steps of a wavefront whose loads are in flight together, as in gemm_skinny_kernel<1, 1, EPI, 4>
+// A quad asks for the first weights of its coming tile while the current one finishes, and, at the end
+// of the phase, for those of its first tile of the next phase: weights do not depend on what the
+// barrier waits for.  `Ahead` carries them.
+#define PROG_U 4  // k steps of a wavefront whose loads are in flight together
 struct Ahead {
-  bf16x8 wf[PROG_U], af[PROG_U];
-  bool has_w, has_a;  // the same in every lane
+  bf16x8 wf[PROG_U];
+  bool has;  // the same in every lane
 };
 
-struct ItemPlace {
-  const bf16_t* wrow;  // this lane's weight row (lane / 4 of the tile, through the rotation's row order if any)
-  int tile, split, k_lo, k_hi;
+// Which tiles of which k range quad `quad` of this workgroup takes: tile first, first + stride, ...
+struct Share {
+  int range, first, stride;
 };
-
-__device__ __forceinline__ ItemPlace place_of(const ProgPhase& ph, int item) {
-  const int lane = threadIdx.x % PAE_WAVE, lrow = lane / 4;
-  const int tiles = (ph.N + 15) / 16;
-  ItemPlace at;
-  at.tile = item % tiles;
-  at.split = item / tiles;
-  at.k_lo = at.split * ph.k_per_split;
-  at.k_hi = min(ph.K, at.k_lo + ph.k_per_split);
-  int n = 16 * at.tile + lrow;
-  if (ph.epilogue == EPI_ROPE) {
-    const int per_head = ph.rope.hd / 16;
-    n = at.tile / per_head * ph.rope.hd + rope_feature(at.tile % per_head, lrow, ph.rope.rot);
+__device__ __forceinline__ Share share_of(int splits, int range_turn, int quad) {
+  const int G = gridDim.x, b = blockIdx.x;
+  Share sh;
+  if (G >= splits) {  // the workgroups whose number is `range` mod splits share the range's tiles
+    sh.range = b % splits;
+    const int rank = b / splits, count = (G - sh.range + splits - 1) / splits;
+    sh.first = rank * PROG_QUADS + quad;
+    sh.stride = count * PROG_QUADS;
+  } else {            // more ranges than workgroups: a workgroup takes whole ranges in turn
+    sh.range = b + range_turn * G;
+    sh.first = quad;
+    sh.stride = PROG_QUADS;
   }
-  at.wrow = ph.W + (int64_t)(n < ph.N ? n : ph.N - 1) * ph.K;  // rows past N are loaded from the last row and never stored
-  return at;
+  return sh;
 }
 
-// The fragments of the PROG_U steps from `kb` on of a row (loads are unconditional, from clamped addresses).
-__device__ __forceinline__ void ask_row(bf16x8 (&frag)[PROG_U], const bf16_t* row, int kb, int K) {
+// This lane's weight row of a tile (row lane / 4, through the rotation's row order if any).
+__device__ __forceinline__ const bf16_t* weight_row(const ProgPhase& ph, int tile) {
+  const int lrow = threadIdx.x % PAE_WAVE / 4;
+  int n = 16 * tile + lrow;
+  if (ph.epilogue == EPI_ROPE) {
+    const int per_head = ph.rope.hd / 16;
+    n = tile / per_head * ph.rope.hd + rope_feature(tile % per_head, lrow, ph.rope.rot);
+  }
+  return ph.W + (int64_t)(n < ph.N ? n : ph.N - 1) * ph.K;  // rows past N are loaded from the last row and never stored
+}
+
+// The weight fragments of the PROG_U steps from `kb` on (loads are unconditional, from clamped addresses).
+__device__ __forceinline__ void ask_weights(bf16x8 (&frag)[PROG_U], const bf16_t* row, int kb, int K) {
   const int lkg = threadIdx.x % 4;
 #pragma unroll
   for (int u = 0; u < PROG_U; ++u) {
@@ -175,119 +185,122 @@ __device__ __forceinline__ void ask_row(bf16x8 (&frag)[PROG_U], const bf16_t* ro
   }
 }
 
-__device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPhase* next, float* quad_lds, int& parity,
-                                              Ahead& ahead) {
+__device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPhase* next, float* quad_lds, bf16x8* a_lds,
+                                              int& parity, Ahead& ahead) {
   const int lane = threadIdx.x % PAE_WAVE;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE), quad = wave / 4, wq = wave % 4;
-  const int M = ph.M, N = ph.N, K = ph.K;
-  const int tiles = (N + 15) / 16, items = tiles * ph.splits, per_round = gridDim.x * PROG_QUADS;
-  const int lrow = lane / 4, g4 = lane / 16;
+  const int M = ph.M, N = ph.N, K = ph.K, splits = ph.splits;
+  const int tiles = (N + 15) / 16;
+  const int g4 = lane / 16;
   const int fetch_from = ((lane % 16) * 4 + lane / 16) * 4;
   constexpr int U = PROG_U, KW = 128, STEP = KW * U;
   float scale[1] = {1.0f};
-  if (wq == 0) row_scales<1>(scale, ph.norm, M, K);  // asked for at once: the shares arrive while the products run
-  const bf16_t* arow = ph.A + (int64_t)(lrow < M ? lrow : M - 1) * ph.lda;
+  if (wq == 0) row_scales<1, true>(scale, ph.norm, M, K);  // asked for at once: the shares arrive while the products run
   const bf16x8 zero = {};
-  struct Batch {
-    bf16x8 wf[U], af[U];
-  };
-  const int first = quad * gridDim.x + blockIdx.x;
-  for (int base = 0; base < items; base += per_round) {
-    const int item = base + first;
-    const bool live = item < items;  // the same in every lane of the quad
-    f32x4 acc[1][1] = {{(f32x4){0.f, 0.f, 0.f, 0.f}}};
-    ItemPlace at = {};
-    if (live) {
-      at = place_of(ph, item);
-      const int k_hi = at.k_hi;
-      auto load = [&](Batch& b, int kb) {
-        ask_row(b.wf, at.wrow, kb, K);
-        ask_row(b.af, arow, kb, K);
-      };
-      auto multiply = [&](Batch& b, int kb) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const bool kok = kb + KW * u + 8 * g4 < k_hi;
-          const bf16x8 a = to_mfma_order(b.af[u], fetch_from);
-          const bf16x8 moved = to_mfma_order(b.wf[u], fetch_from);
-          acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kok ? moved : zero, a, acc[0][0], 0, 0, 0);
-        }
-      };
-      int kb = at.k_lo + 32 * wq;
-      Batch b0, b1;
-      if (kb < k_hi) {
-        if (ahead.has_w) {
-#pragma unroll
-          for (int u = 0; u < U; ++u) b0.wf[u] = ahead.wf[u];
-        } else {
-          ask_row(b0.wf, at.wrow, kb, K);
-        }
-        if (ahead.has_a) {
-#pragma unroll
-          for (int u = 0; u < U; ++u) b0.af[u] = ahead.af[u];
-        } else {
-          ask_row(b0.af, arow, kb, K);
-        }
-      }
-      ahead.has_w = ahead.has_a = false;
-      // the coming round's item, asked for as soon as this item's last loads are out
-      bool asked = false;
-      auto ask_ahead = [&]() {
-        asked = true;
-        if (item + per_round < items) {
-          const ItemPlace then = place_of(ph, item + per_round);
-          ask_row(ahead.wf, then.wrow, then.k_lo + 32 * wq, K);
-          ask_row(ahead.af, arow, then.k_lo + 32 * wq, K);
-          ahead.has_w = ahead.has_a = true;
-        }
-      };
-      while (kb < k_hi) {
-        if (kb + STEP < k_hi) load(b1, kb + STEP);
-        else if (!asked) ask_ahead();
-        multiply(b0, kb);
-        kb += STEP;
-        if (kb >= k_hi) break;
-        if (kb + STEP < k_hi) load(b0, kb + STEP);
-        else if (!asked) ask_ahead();
-        multiply(b1, kb);
-        kb += STEP;
-      }
-      if (!asked) ask_ahead();
-    }
-    float* s_part = quad_lds + parity * (3 * 4 * PAE_WAVE);  // [3][4][64]
-    parity ^= 1;
-    if (live && wq > 0) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) s_part[((wq - 1) * 4 + i) * PAE_WAVE + lane] = acc[0][0][i];
+  const int range_turns = gridDim.x >= splits ? 1 : (splits - blockIdx.x + gridDim.x - 1) / gridDim.x;
+  for (int turn = 0; turn < range_turns; ++turn) {
+    const Share sh = share_of(splits, turn, quad);
+    const int k_lo = sh.range * ph.k_per_split, k_hi = min(K, k_lo + ph.k_per_split);
+    // the range's activations: chunk c of row m (8 elements at k_lo + 8 c) is what lane 16 (c % 4) + m of
+    // k step c / 4 multiplies; the last step's chunks past the range are zero (their weights are zeroed
+    // too, but zero times whatever LDS held is not always zero)
+    const int chunks = (k_hi - k_lo) / 8, padded = (chunks + 3) / 4 * 4;
+    if (turn > 0) __syncthreads();  // the range before has been read
+    for (int idx = threadIdx.x; idx < M * padded; idx += PROG_THREADS) {
+      const int m = idx / padded, c = idx % padded;
+      bf16x8 v = zero;
+      if (c < chunks) v = load_through(reinterpret_cast<const bf16x8*>(ph.A + (int64_t)m * ph.lda + k_lo + 8 * c));
+      a_lds[(c / 4) * PAE_WAVE + (c % 4) * 16 + m] = v;
     }
     __syncthreads();
-    if (!live || wq > 0) continue;
+    for (int base = 0; base < tiles; base += sh.stride) {
+      const int tile = base + sh.first;
+      const bool live = tile < tiles;  // the same in every lane of the quad
+      f32x4 acc[1][1] = {{(f32x4){0.f, 0.f, 0.f, 0.f}}};
+      if (live) {
+        const bf16_t* wrow = weight_row(ph, tile);
+        auto multiply = [&](bf16x8 (&wf)[U], int kb) {
 #pragma unroll
-    for (int w = 0; w < 3; ++w)
+          for (int u = 0; u < U; ++u) {
+            const int k = kb + KW * u;  // this wavefront's step: k .. k + 31
+            const bool kok = k + 8 * g4 < k_hi;
+            // (past the range the step's place in LDS is the last one's: its weights are zero)
+            const bf16x8 a = a_lds[(min(k, k_hi - 1) - k_lo) / 32 * PAE_WAVE + lane];
+            const bf16x8 moved = to_mfma_order(wf[u], fetch_from);
+            acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kok ? moved : zero, a, acc[0][0], 0, 0, 0);
+          }
+        };
+        int kb = k_lo + 32 * wq;
+        bf16x8 w0[U], w1[U];
+        if (kb < k_hi) {
+          if (ahead.has) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[0][0][i] += s_part[(w * 4 + i) * PAE_WAVE + lane];
-    if (ph.epilogue != EPI_F32 && ph.splits > 1) {
-      f32x4 mine[1] = {acc[0][0]};
-      if (!add_up_k_ranges<1>(mine, at.tile, at.split, ph.splits, SkinnyTickets{ph.ticket_parts, ph.ticket_counters})) continue;
-      acc[0][0] = mine[0];
-    }
+            for (int u = 0; u < U; ++u) w0[u] = ahead.wf[u];
+          } else {
+            ask_weights(w0, wrow, kb, K);
+          }
+        }
+        ahead.has = false;
+        // the coming round's tile, asked for as soon as this tile's last loads are out
+        bool asked = false;
+        auto ask_ahead = [&]() {
+          asked = true;
+          if (tile + sh.stride < tiles) {
+            ask_weights(ahead.wf, weight_row(ph, tile + sh.stride), k_lo + 32 * wq, K);
+            ahead.has = true;
+          }
+        };
+        while (kb < k_hi) {
+          if (kb + STEP < k_hi) ask_weights(w1, wrow, kb + STEP, K);
+          else if (!asked) ask_ahead();
+          multiply(w0, kb);
+          kb += STEP;
+          if (kb >= k_hi) break;
+          if (kb + STEP < k_hi) ask_weights(w0, wrow, kb + STEP, K);
+          else if (!asked) ask_ahead();
+          multiply(w1, kb);
+          kb += STEP;
+        }
+        if (!asked) ask_ahead();
+      }
+      float* s_part = quad_lds + parity * (3 * 4 * PAE_WAVE);  // [3][4][64]
+      parity ^= 1;
+      if (live && wq > 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_part[((wq - 1) * 4 + i) * PAE_WAVE + lane] = acc[0][0][i];
+      }
+      __syncthreads();
+      if (!live || wq > 0) continue;
+#pragma unroll
+      for (int w = 0; w < 3; ++w)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[0][0][i] += s_part[(w * 4 + i) * PAE_WAVE + lane];
+      if (ph.epilogue != EPI_F32 && splits > 1) {
+        f32x4 mine[1] = {acc[0][0]};
+        if (!add_up_k_ranges<1>(mine, tile, sh.range, splits, SkinnyTickets{ph.ticket_parts, ph.ticket_counters})) continue;
+        acc[0][0] = mine[0];
+      }
 #define PROG_EPILOGUE(EPI)                                                                                          \
-  skinny_epilogue<1, 1, EPI, true>(acc, at.tile, -1, ph.out, ph.ldc, ph.bias, ph.b_is_f32, M, N, at.split, (int64_t)M * N, \
+  skinny_epilogue<1, 1, EPI, true>(acc, tile, -1, ph.out, ph.ldc, ph.bias, ph.b_is_f32, M, N, sh.range, (int64_t)M * N, \
                                    ph.rope, ph.norm, scale)
-    switch (ph.epilogue) {  // the one place where the epilogues part ways: the products above are the same code for all
-      case EPI_BF16: PROG_EPILOGUE(EPI_BF16); break;
-      case EPI_F32: PROG_EPILOGUE(EPI_F32); break;
-      case EPI_SWIGLU: PROG_EPILOGUE(EPI_SWIGLU); break;
-      case EPI_ROPE: PROG_EPILOGUE(EPI_ROPE); break;
-      default: PROG_EPILOGUE(EPI_RESIDUAL); break;
-    }
+      switch (ph.epilogue) {  // the one place where the epilogues part ways: the products above are the same code for all
+        case EPI_BF16: PROG_EPILOGUE(EPI_BF16); break;
+        case EPI_F32: PROG_EPILOGUE(EPI_F32); break;
+        case EPI_SWIGLU: PROG_EPILOGUE(EPI_SWIGLU); break;
+        case EPI_ROPE: PROG_EPILOGUE(EPI_ROPE); break;
+        default: PROG_EPILOGUE(EPI_RESIDUAL); break;
+      }
 #undef PROG_EPILOGUE
+    }
   }
-  // the weights of this quad's first item of the next phase, on their way while the barrier is crossed
-  if (!ahead.has_w && next && next->type == PROG_PRODUCT && first < (next->N + 15) / 16 * next->splits) {
-    const ItemPlace then = place_of(*next, first);
-    ask_row(ahead.wf, then.wrow, then.k_lo + 32 * wq, next->K);
-    ahead.has_w = true;
+  // the weights of this quad's first tile of the next phase, on their way while the barrier is crossed
+  ahead.has = false;
+  if (next && next->type == PROG_PRODUCT) {
+    const Share then = share_of(next->splits, 0, quad);
+    if (then.range < next->splits && then.first < (next->N + 15) / 16) {
+      ask_weights(ahead.wf, weight_row(*next, then.first), then.range * next->k_per_split + 32 * wq, next->K);
+      ahead.has = true;
+    }
   }
 }
 
@@ -297,6 +310,24 @@ __device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPha
 // attn_decode_kernel's workgroup; it then leaves its partial result in memory and draws a ticket
 // from the (token, head)'s counter, and the quad that draws the last one merges all of the splits:
 // its four wavefronts are attn_decode_merge_kernel's four groups of splits.
+//
+// The queries, the page that holds the token's own key and value (written by the phase before) and
+// the partial results are read with device-scope loads; every other page has not been written since
+// the kernel began and is read plainly.
+template <int HD>
+__device__ __forceinline__ void load_kv_tile_through(bf16x8 (&kf)[HD / 32], s16x4 (&vf)[HD / 16], const bf16_t* kp,
+                                                     const bf16_t* vp, int vstride) {
+  const int lane = threadIdx.x % PAE_WAVE;
+  const int r = lane / 4, g = lane % 4;
+#pragma unroll
+  for (int j = 0; j < HD / 32; ++j) kf[j] = load_through(reinterpret_cast<const bf16x8*>(kp + r * HD + 32 * j + 8 * g));
+#pragma unroll
+  for (int t = 0; t < HD / 16; ++t)
+    vf[t] = load_through(reinterpret_cast<const s16x4*>(vp + (int64_t)(16 * t + lane % 16) * vstride + 4 * (lane / 16)));
+}
+
+#define PROG_MERGE_BATCH 16  // splits of one wavefront whose partial results are in flight together
+
 template <int HD>
 __device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad_lds, int* s_flag) {
   constexpr int TPW = PROG_SPLIT / 64, ROWS = HD / 4 + 2;
@@ -326,16 +357,7 @@ __device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad
       const int lo = max(split * PROG_SPLIT, start[0] / 16 * 16);
       const int hi = min((split + 1) * PROG_SPLIT, pos[0] + 1);
       const int* table = ph.block_tables + (int64_t)work.z * ph.max_blocks;
-      bf16x8 qf[1][HD / 32];
-      const bf16_t* qrow = ph.q + (int64_t)work.x * ph.q_stride + (int64_t)(kvh * g + (col < g ? col : 0)) * HD;
-#pragma unroll
-      for (int j = 0; j < HD / 32; ++j) {
-        qf[0][j] = *reinterpret_cast<const bf16x8*>(qrow + 32 * j + 8 * g4);
-        if (col >= g)
-#pragma unroll
-          for (int e = 0; e < 8; ++e) qf[0][j][e] = (__bf16)0.f;
-      }
-      const int tile_lo = lo / 16, tile_hi = (hi + 15) / 16;
+      const int tile_lo = lo / 16, tile_hi = (hi + 15) / 16, own_tile = pos[0] / 16;
       bf16x8 kf[TPW][HD / 32];
       s16x4 vf[TPW][HD / 16];
 #pragma unroll
@@ -343,7 +365,19 @@ __device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad
         const int tile = tile_lo + wq + 4 * j;
         const int key0 = (tile < tile_hi ? tile : tile_lo) * 16;
         const int64_t at = ((int64_t)table[key0 / bs] * nkv + kvh) * page_elems;
-        load_kv_tile<HD>(kf[j], vf[j], ph.k_cache + at + (int64_t)(key0 % bs) * HD, ph.v_cache + at + key0 % bs, bs);
+        const bf16_t* kp = ph.k_cache + at + (int64_t)(key0 % bs) * HD;
+        const bf16_t* vp = ph.v_cache + at + key0 % bs;
+        if (key0 / 16 == own_tile) load_kv_tile_through<HD>(kf[j], vf[j], kp, vp, bs);  // the same in the whole wavefront
+        else load_kv_tile<HD>(kf[j], vf[j], kp, vp, bs);
+      }
+      bf16x8 qf[1][HD / 32];
+      const bf16_t* qrow = ph.q + (int64_t)work.x * ph.q_stride + (int64_t)(kvh * g + (col < g ? col : 0)) * HD;
+#pragma unroll
+      for (int j = 0; j < HD / 32; ++j) {
+        qf[0][j] = load_through(reinterpret_cast<const bf16x8*>(qrow + 32 * j + 8 * g4));
+        if (col >= g)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) qf[0][j][e] = (__bf16)0.f;
       }
 #pragma unroll
       for (int j = 0; j < TPW; ++j) {
@@ -410,33 +444,41 @@ __device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad
     if (!any) continue;
     const int pair = s_flag[quad];
     // the merging quad: wavefront w adds the splits s_first + w, + 4, ... of every (head, four features)
-    // in split order (loads of eight splits in flight together) and leaves its sums in LDS
-    int m_first = 0, m_count = 0, m_tok = 0, m_kvh = 0;
+    // in split order, PROG_MERGE_BATCH of them in flight together, and leaves its sums in LDS
+    int m_tok = 0, m_kvh = 0;
     if (pair >= 0) {
       const int4 mw = ph.dec_work[pair / nkv];
       m_tok = mw.x;
       m_kvh = pair % nkv;
       const int mstart = (window > 0 && mw.y - window + 1 > 0) ? mw.y - window + 1 : 0;
-      m_first = mstart / PROG_SPLIT;
-      m_count = mw.y / PROG_SPLIT - m_first + 1;
-      // the partials were written through by quads of any die while this die's L2 may still hold what
-      // an earlier step left at their addresses
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      const int m_first = mstart / PROG_SPLIT, m_count = mw.y / PROG_SPLIT - m_first + 1;
       for (int it = lane; it < merge_items; it += PAE_WAVE) {
         const int c = it / (HD / 4), d = (it % (HD / 4)) * 4;
         const int64_t slot0 = ((int64_t)pair * max_splits + m_first) * g + c;
         float m = NEG_BIG, l = 0.f;
         f32x4 a = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 8
-        for (int sp = wq; sp < m_count; sp += 4) {
-          const int64_t slot = slot0 + (int64_t)sp * g;
-          const float ms = ph.part_ml[slot * 2], ls = ph.part_ml[slot * 2 + 1];
-          const f32x4 v = *reinterpret_cast<const f32x4*>(ph.part_acc + slot * HD + d);
-          const float m_new = fmaxf(m, ms);
-          const float f_old = exp2f(m - m_new), f = exp2f(ms - m_new);
-          a = a * f_old + v * f;
-          l = l * f_old + ls * f;
-          m = m_new;
+        for (int sp0 = wq; sp0 < m_count; sp0 += 4 * PROG_MERGE_BATCH) {
+          f32x4 v[PROG_MERGE_BATCH];
+          float ms[PROG_MERGE_BATCH], ls[PROG_MERGE_BATCH];
+#pragma unroll
+          for (int j = 0; j < PROG_MERGE_BATCH; ++j) {
+            const int sp = sp0 + 4 * j;
+            const int64_t slot = slot0 + (int64_t)(sp < m_count ? sp : sp0) * g;  // past the end: the batch's first, not used
+            v[j] = load_through(reinterpret_cast<const f32x4*>(ph.part_acc + slot * HD + d));
+            const unsigned long long raw = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(ph.part_ml + slot * 2),
+                                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ms[j] = __uint_as_float((unsigned)raw);
+            ls[j] = __uint_as_float((unsigned)(raw >> 32));
+          }
+#pragma unroll
+          for (int j = 0; j < PROG_MERGE_BATCH; ++j) {
+            if (sp0 + 4 * j >= m_count) break;
+            const float m_new = fmaxf(m, ms[j]);
+            const float f_old = exp2f(m - m_new), f = exp2f(ms[j] - m_new);
+            a = a * f_old + v[j] * f;
+            l = l * f_old + ls[j] * f;
+            m = m_new;
+          }
         }
         float* dst = quad_lds + ((int64_t)wq * merge_items + it) * 6;
         dst[0] = a[0]; dst[1] = a[1]; dst[2] = a[2]; dst[3] = a[3]; dst[4] = m; dst[5] = l;
@@ -471,7 +513,10 @@ __device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad
 
 __global__ __launch_bounds__(PROG_THREADS) void decode_program_kernel(const ProgPhase* phases, int num_phases,
                                                                       ProgBarrier* bar, int* host_error,
-                                                                      int quad_floats, int spin_limit) {
+                                                                      int quad_floats, int spin_limit,
+                                                                      long long* trace) {
+  // dynamic LDS: the quads' regions (sums of a quad's wavefronts, attention states, merges), then the
+  // region for a product's activations
   extern __shared__ float s_mem[];
   __shared__ int s_flag[PROG_QUADS];
   __shared__ int s_dead;
@@ -488,6 +533,7 @@ __global__ __launch_bounds__(PROG_THREADS) void decode_program_kernel(const Prog
     if (threadIdx.x < PIECES) reinterpret_cast<int4*>(&s_phase[p % 3])[threadIdx.x] = piece;
   };
   float* quad_lds = s_mem + (int64_t)(threadIdx.x / (4 * PAE_WAVE)) * quad_floats;
+  bf16x8* a_lds = reinterpret_cast<bf16x8*>(s_mem + (int64_t)PROG_QUADS * quad_floats);
   unsigned epoch = 0;
   if (threadIdx.x == 0) {
     s_dead = 0;
@@ -504,18 +550,20 @@ __global__ __launch_bounds__(PROG_THREADS) void decode_program_kernel(const Prog
   __syncthreads();
   int parity = 0;
   Ahead ahead;
-  ahead.has_w = ahead.has_a = false;
+  ahead.has = false;
   for (int p = 0; p < num_phases; ++p) {
     const ProgPhase& ph = s_phase[p % 3];
     const ProgPhase* next = p + 1 < num_phases ? &s_phase[(p + 1) % 3] : nullptr;
     if (p + 2 < num_phases) ask_for_phase(p + 2);  // kept when this phase is over
+    if (trace && threadIdx.x == 0) trace[((int64_t)p * gridDim.x + blockIdx.x) * 2] = wall_clock64();
     if (ph.type == PROG_PRODUCT) {
-      product_phase(ph, next, quad_lds, parity, ahead);
+      product_phase(ph, next, quad_lds, a_lds, parity, ahead);
     } else {
       if (ph.hd == 128) attention_phase<128>(ph, quad_lds, s_flag);
       else attention_phase<64>(ph, quad_lds, s_flag);
       ahead = Ahead{};  // nothing is carried across an attention phase (and the registers are free during it)
     }
+    if (trace && threadIdx.x == 0) trace[((int64_t)p * gridDim.x + blockIdx.x) * 2 + 1] = wall_clock64();
     if (p + 1 == num_phases) break;
     // into the buffer of phase p - 1, whose last readers passed the barrier's workgroup barriers a phase ago
     if (p + 2 < num_phases) keep_phase(p + 2);
@@ -532,6 +580,17 @@ extern "C" int pae_program_barrier_bytes() { return (int)sizeof(ProgBarrier); }
 extern "C" int pae_program_max_rows() { return PROG_MAX_ROWS; }
 
 static int quad_bytes_of_product() { return 2 * 3 * 4 * PAE_WAVE * (int)sizeof(float); }
+
+// Bytes of LDS that the activations of one k range of a product take in a workgroup: `rows` rows of one
+// range, whole k steps of 32.
+extern "C" int pae_program_activation_bytes(int rows, int K, int splits) {
+  if (rows < 1 || K < 1 || splits < 1) return 0;
+  int k_per_split = (K + splits - 1) / splits;
+  k_per_split = (k_per_split + 127) / 128 * 128;
+  if (k_per_split > K) k_per_split = (K + 31) / 32 * 32;
+  return k_per_split / 32 * PAE_WAVE * 16;
+}
+extern "C" int pae_program_lds_limit();
 
 // Writes phase `index` of the host-side list `phases`: a product with any epilogue but the rotating
 // one.  Arguments as pae_gemm_skinny; the k ranges are those that call would take.  Returns the
@@ -635,6 +694,8 @@ extern "C" int pae_program_put_attention(void* phases, int index, void* out, int
 #define PROG_LDS_LIMIT (160 * 1024 - 2048)  // dynamic LDS: what the kernel declares for itself (phase descriptions, flags) stays below 2 KB
 static int g_max_groups[64];
 
+extern "C" int pae_program_lds_limit() { return PROG_LDS_LIMIT; }
+
 extern "C" int pae_program_max_groups() {
   int dev = 0, units = 0, per_unit = 0;
   hipError_t err = hipGetDevice(&dev);
@@ -656,12 +717,16 @@ extern "C" int pae_program_max_groups() {
 // pae_program_barrier_bytes() of device memory, zero before its first use and used with one value of
 // `groups` only; `host_error` is an int in pinned host memory that receives 1 + the phase at whose
 // barrier a workgroup gave up after `spin_limit` polls (it stays as it is otherwise).  Launches that
-// share a barrier block or ticket counters must not overlap.
+// share a barrier block or ticket counters must not overlap.  `trace` (or null): device memory for
+// num_phases * groups * 2 clock readings (100 MHz), when every workgroup began and ended every phase.
 extern "C" int pae_program_run(const void* phases, int num_phases, void* barrier, int* host_error, int groups,
-                               int quad_lds_bytes, int spin_limit, hipStream_t stream) {
+                               int quad_lds_bytes, int activation_lds_bytes, int spin_limit, long long* trace,
+                               hipStream_t stream) {
   PAE_REQUIRE(phases && barrier && host_error && num_phases >= 1, "decode program: nothing to run");
-  PAE_REQUIRE(quad_lds_bytes >= quad_bytes_of_product() && quad_lds_bytes % 16 == 0 && quad_lds_bytes * PROG_QUADS <= PROG_LDS_LIMIT,
-              "decode program: %d bytes of LDS a quad", quad_lds_bytes);
+  PAE_REQUIRE(quad_lds_bytes >= quad_bytes_of_product() && quad_lds_bytes % 16 == 0 && activation_lds_bytes >= 0 &&
+              activation_lds_bytes % 16 == 0 && (int64_t)quad_lds_bytes * PROG_QUADS + activation_lds_bytes <= PROG_LDS_LIMIT,
+              "decode program: %d bytes of LDS a quad and %d for a product's activations exceed the %d there are",
+              quad_lds_bytes, activation_lds_bytes, PROG_LDS_LIMIT);
   PAE_REQUIRE(spin_limit > 0, "decode program: the waits must be bounded");
   int dev = 0;
   PAE_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && g_max_groups[dev] > 0,
@@ -669,7 +734,8 @@ extern "C" int pae_program_run(const void* phases, int num_phases, void* barrier
   // every workgroup must be resident at once, or the barrier between the phases never completes
   PAE_REQUIRE(groups >= 1 && groups <= g_max_groups[dev], "decode program: %d workgroups cannot all be resident (at most %d)",
               groups, g_max_groups[dev]);
-  decode_program_kernel<<<groups, PROG_THREADS, (size_t)quad_lds_bytes * PROG_QUADS, stream>>>(
-      (const ProgPhase*)phases, num_phases, (ProgBarrier*)barrier, host_error, quad_lds_bytes / (int)sizeof(float), spin_limit);
+  decode_program_kernel<<<groups, PROG_THREADS, (size_t)quad_lds_bytes * PROG_QUADS + activation_lds_bytes, stream>>>(
+      (const ProgPhase*)phases, num_phases, (ProgBarrier*)barrier, host_error, quad_lds_bytes / (int)sizeof(float), spin_limit,
+      trace);
   return pae_check_launch("decode program");
 }

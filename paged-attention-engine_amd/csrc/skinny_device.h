@@ -37,11 +37,34 @@ struct SkinnyNorm {
   float* next_stats;       // [M][(N + 15) / 16]
 };
 
+// Loads that see what another die has written through during the same kernel (device-scope loads are
+// served past the die's own L2, which may hold an older copy of the line); see `put` and SkinnyTickets below.
+__device__ __forceinline__ float load_through(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f32x4 load_through(const f32x4* p) {
+  unsigned long long raw[2];
+  raw[0] = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  raw[1] = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return *reinterpret_cast<f32x4*>(raw);
+}
+__device__ __forceinline__ bf16x8 load_through(const bf16x8* p) {
+  unsigned long long raw[2];
+  raw[0] = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  raw[1] = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return *reinterpret_cast<bf16x8*>(raw);
+}
+__device__ __forceinline__ s16x4 load_through(const s16x4* p) {
+  unsigned long long raw = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return *reinterpret_cast<s16x4*>(&raw);
+}
+
 // rsqrt(mean of squares + eps) of row m of A from the shares the producer left.  The four lanes
 // that hold row m (g4 = 0..3) read the shares 16 bytes at a time, all reads of a batch of up to
 // 128 shares in flight at once (a loop that adds one share after the other waits out the memory's
 // latency once per share), add theirs in index order and then each other's: the same order in every
 // workgroup, so every column of a row is scaled by the same number.
+template <bool THROUGH = false>
 __device__ __forceinline__ float row_scale_of(const SkinnyNorm& norm, int m, int g4, float inv_width) {
   const float* shares = norm.row_stats + (int64_t)m * norm.row_stat_tiles;
   const int tiles = norm.row_stat_tiles;
@@ -53,10 +76,10 @@ __device__ __forceinline__ float row_scale_of(const SkinnyNorm& norm, int m, int
     for (int u = 0; u < 8; ++u) {
       const int t = base + 16 * u + 4 * g4;
       if (aligned && t + 4 <= tiles) {
-        part[u] = *reinterpret_cast<const f32x4*>(shares + t);
+        part[u] = THROUGH ? load_through(reinterpret_cast<const f32x4*>(shares + t)) : *reinterpret_cast<const f32x4*>(shares + t);
       } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) part[u][i] = t + i < tiles ? shares[t + i] : 0.f;
+        for (int i = 0; i < 4; ++i) part[u][i] = t + i < tiles ? (THROUGH ? load_through(shares + t + i) : shares[t + i]) : 0.f;
       }
     }
 #pragma unroll
@@ -69,13 +92,13 @@ __device__ __forceinline__ float row_scale_of(const SkinnyNorm& norm, int m, int
 
 // The scales of this lane's rows of A (row 16 mt + lane % 16 of column tile mt), 1 without a folded
 // norm.  Asked for at the start of a kernel, so that the shares arrive while the products run.
-template <int MT>
+template <int MT, bool THROUGH = false>
 __device__ __forceinline__ void row_scales(float (&scale)[MT], const SkinnyNorm& norm, int M, int K) {
   const int lane = threadIdx.x % PAE_WAVE;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + lane % 16;
-    scale[mt] = norm.row_stats ? row_scale_of(norm, m < M ? m : M - 1, lane / 16, 1.0f / (float)K) : 1.0f;
+    scale[mt] = norm.row_stats ? row_scale_of<THROUGH>(norm, m < M ? m : M - 1, lane / 16, 1.0f / (float)K) : 1.0f;
   }
 }
 
@@ -243,7 +266,7 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const bool in = n + i < N;
-            v[i] = in ? res[n + i] + acc[rt][mt][i] * scale[mt] : 0.f;
+            v[i] = in ? (THROUGH ? load_through(res + n + i) : res[n + i]) + acc[rt][mt][i] * scale[mt] : 0.f;
             ss += v[i] * v[i];
             p[i] = to_bf16_bits(in ? v[i] * load_param(norm.next_w, norm.next_w_is_f32, n + i) : 0.f);
           }

@@ -85,7 +85,9 @@ def _declare(lib) -> None:
         "pae_program_put_product_rope": [P, I, P, L, P, L, P, P, I, I, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P, P, P,
                                          I, F],
         "pae_program_put_attention": [P, I, P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, P, P, P],
-        "pae_program_run": [P, I, P, P, I, I, I, P],
+        "pae_program_run": [P, I, P, P, I, I, I, I, P, P],
+        "pae_program_activation_bytes": [I, I, I],
+        "pae_program_lds_limit": [],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -314,6 +316,13 @@ def program_max_rows() -> int:
     return library().pae_program_max_rows()
 
 
+def program_takes_product(rows: int, K: int, splits: int, quad_bytes: int = 27 * 1024) -> bool:
+    """Whether a decode program has the LDS for a product of `rows` rows over k ranges of K / splits
+    (a workgroup keeps one range's activations there, beside its quads' own `quad_bytes` each)."""
+    lib = library()
+    return 2 * quad_bytes + lib.pae_program_activation_bytes(rows, K, splits) <= lib.pae_program_lds_limit()
+
+
 _PROGRAM_BARRIERS: dict = {}  # (device index, workgroups) -> zeroed barrier block
 
 
@@ -347,23 +356,27 @@ class DecodeProgram:
         skinny_tickets(self.device)
         self.host_ptr = self.host.data_ptr()
         self.count = 0
-        self.quad_lds = 0
+        self.quad_lds = 0        # bytes of LDS a quad needs: the most any phase asked for
+        self.activation_lds = 0  # bytes of LDS for a product's activations: likewise
         self.keep: list = []
         self._read: Optional[torch.cuda.Event] = None
+        self.trace: Optional[torch.Tensor] = None  # int64 [phases, workgroups, 2] clock readings of the next launches, if set
 
     def begin(self) -> None:
         if self._read is not None:
             self._read.synchronize()  # the launch before has copied the list to the device
-        self.count, self.quad_lds, self.keep = 0, 0, []
+        self.count, self.quad_lds, self.activation_lds, self.keep = 0, 0, 0, []
 
-    def add(self, code: int, *tensors) -> None:
-        """`code`: what a pae_program_put_* call returned (the bytes of LDS a quad needs, or an error)."""
+    def add(self, code: int, *tensors, activation_bytes: int = 0) -> None:
+        """`code`: what a pae_program_put_* call returned (the bytes of LDS a quad needs, or an error);
+        `activation_bytes`: the LDS a product's activations take (pae_program_activation_bytes)."""
         if code < 0:
             _check(code)
         if self.count + 1 > self.max_phases:
             raise KernelError(f"a decode program of more than {self.max_phases} phases")
         self.count += 1
         self.quad_lds = max(self.quad_lds, code)
+        self.activation_lds = max(self.activation_lds, activation_bytes)
         self.keep.append(tensors)  # what the phase reads and writes stays alive until the program has run
 
     def launch(self) -> None:
@@ -373,10 +386,17 @@ class DecodeProgram:
         assert _RECORDING is None, "a program is launched after its recording has ended"
         copy_int32_from_pinned(self.on_device, self.host, self.count * self.phase_bytes // 4)
         _check(library().pae_program_run(self.on_device.data_ptr(), self.count, self.barrier.data_ptr(),
-                                         self.error.data_ptr(), self.groups, self.quad_lds, PROGRAM_SPIN_LIMIT, _stream()))
+                                         self.error.data_ptr(), self.groups, self.quad_lds, self.activation_lds,
+                                         PROGRAM_SPIN_LIMIT, _ptr(self.trace), _stream()))
         if not torch.cuda.is_current_stream_capturing():
             self._read = self._read or torch.cuda.Event()
             self._read.record()
+
+    def trace_phases(self) -> torch.Tensor:
+        """From now on every launch leaves, per phase and workgroup, the clock (100 MHz) at which it began
+        and ended the phase's work (the difference to the next phase's beginning is its wait at the barrier)."""
+        self.trace = torch.zeros((self.max_phases, self.groups, 2), dtype=torch.int64, device=self.device)
+        return self.trace
 
     def check(self) -> None:
         """Raise if a launch of this program gave up at a barrier (call after the device has been waited for)."""
@@ -558,7 +578,8 @@ def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optio
         _RECORDING.add(library().pae_program_put_product(
             _RECORDING.host_ptr, _RECORDING.count, epilogue, out.data_ptr(), out.stride(-2), a.data_ptr(), a.stride(0),
             w.data_ptr(), bp, bf, M, N, K_, splits, _ptr(parts), _ptr(counters), sp, st, se, nr, ld_next, nw, nwf, ns,
-            None), out, a, w, bias, parts, row_scale, following)
+            None), out, a, w, bias, parts, row_scale, following,
+            activation_bytes=library().pae_program_activation_bytes(M, K_, splits))
         return
     checking = (parts is not None and CHECK_TICKET_SUMS and not torch.cuda.is_current_stream_capturing())
     before = out.clone() if checking and epilogue == EPI_RESIDUAL else None
@@ -724,7 +745,8 @@ def gemm_skinny_rope(q_out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias
             _RECORDING.host_ptr, _RECORDING.count, q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0),
             w.data_ptr(), bp, bf, M, K_, nh, nkv, hd, rot, _ptr(cos_sin) if rot else None, positions.data_ptr(),
             _ptr(tok_seq), _ptr(block_tables), max_blocks, block_size, _ptr(k_cache), _ptr(v_cache), splits, _ptr(parts),
-            _ptr(counters), sp, st, se), q_out, a, w, bias, cos_sin, parts, row_scale)
+            _ptr(counters), sp, st, se), q_out, a, w, bias, cos_sin, parts, row_scale,
+            activation_bytes=lib.pae_program_activation_bytes(M, K_, splits))
         return
     _launch_ticketed(counters, lambda: lib.pae_gemm_skinny_rope(
         q_out.data_ptr(), q_out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(), bp, bf, M, K_, nh, nkv, hd, rot,

@@ -78,7 +78,11 @@ class PagedAttention(Part):
         return (self.dtype == torch.bfloat16 and 0 < rows <= K.program_max_rows() and self._matrix_cores(block_size)
                 and s.head_dim in (64, 128) and group * s.head_dim <= 1024 and not s.out_bias
                 and hasattr(self.position, "rotary_table") and s.hidden_size % 8 == 0
-                and getattr(s.position, "rotary_dim", 0) % 16 == 0)
+                and getattr(s.position, "rotary_dim", 0) % 16 == 0
+                and K.program_takes_product(rows, s.hidden_size, K.whole_sum_splits(
+                    (s.num_heads + 2 * s.num_kv_heads) * s.head_dim, s.hidden_size, rows))
+                and K.program_takes_product(rows, s.num_heads * s.head_dim, K.residual_splits(
+                    s.hidden_size, s.num_heads * s.head_dim, rows)))
 
     def paged_spec(self):
         return attention_pages(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)

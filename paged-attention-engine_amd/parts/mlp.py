@@ -49,7 +49,11 @@ class SwiGLU(Part):
     def decode_fusable(self, rows: int, block_size: int) -> bool:
         s = self.spec
         return (self.dtype == torch.bfloat16 and bool(self.block) and 0 < rows <= K.program_max_rows()
-                and s.hidden_size % 8 == 0 and s.intermediate_size % 8 == 0)
+                and s.hidden_size % 8 == 0 and s.intermediate_size % 8 == 0
+                and K.program_takes_product(rows, s.hidden_size,
+                                            K.whole_sum_splits(2 * s.intermediate_size, s.hidden_size, rows))
+                and K.program_takes_product(rows, s.intermediate_size,
+                                            K.residual_splits(s.hidden_size, s.intermediate_size, rows)))
 
     def forward(self, ctx, x):
         """`x`: normalised activations, or `OwedRows` (the gated product then pays their scale)."""
