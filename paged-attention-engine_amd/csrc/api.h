@@ -57,6 +57,35 @@ int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t 
                           const void* v_cache, const int* tiles, int num_tiles, const int* positions,
                           const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,
                           int window, hipStream_t stream);
+// A decode step's layers as one resident kernel (see decode_program.hip).
+// A caller builds a list of phases in host memory with the put functions (each returns the bytes of
+// LDS a quad of four wavefronts needs for the phase, or a negative code), copies it to the device and
+// runs it.  pae_program_max_groups() must have been called once on the device, outside any capture.
+struct SkinnyRope;
+int pae_program_phase_bytes();
+int pae_program_barrier_bytes();
+int pae_program_max_rows();
+int pae_program_max_groups();
+int pae_program_lds_limit();
+int pae_program_activation_bytes(int rows, int K, int splits);
+int pae_program_put_product(void* phases, int index, int epilogue, void* out, int64_t ldc, const void* A, int64_t lda,
+                            const void* W, const void* bias, int b_is_f32, int M, int N, int K, int splits,
+                            float* ticket_parts, int* ticket_counters, const float* row_stats, int row_stat_tiles,
+                            float row_eps, void* next_rows, int64_t ld_next, const void* next_w, int next_w_is_f32,
+                            float* next_stats, const SkinnyRope* rope);
+int pae_program_put_product_rope(void* phases, int index, void* q_out, int64_t ldq, const void* A, int64_t lda,
+                                 const void* W, const void* bias, int b_is_f32, int M, int K, int nh, int nkv, int hd,
+                                 int rot, const float* cos_sin, const int* positions, const int* tok_seq,
+                                 const int* block_tables, int max_blocks, int bs, void* k_cache, void* v_cache,
+                                 int splits, float* ticket_parts, int* ticket_counters, const float* row_stats,
+                                 int row_stat_tiles, float row_eps);
+int pae_program_put_attention(void* phases, int index, void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                              const void* k_cache, const void* v_cache, const int* dec_work, int num_dec,
+                              const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,
+                              int window, void* part_acc, void* part_ml, int* ticket_counters);
+int pae_program_run(const void* phases, int num_phases, void* barrier, int* host_error, int groups, int quad_lds_bytes,
+                    int activation_lds_bytes, int spin_limit, long long* trace, hipStream_t stream);
+
 int pae_sample_chunks(int vocab);
 int pae_sample(int* tokens, const float* logits, int64_t ld, const float* temperature, const float* uniform,
                int num_rows, int vocab, float* chunk_max, int* chunk_arg, double* chunk_sum, hipStream_t stream);

@@ -430,7 +430,9 @@ class recording:
 
 
 SKINNY_MAX_ROWS = 64
-FOLD_MAX_ROWS = 16  # up to this many rows a norm is folded into the products around it (see parts.OwedRows)
+# up to this many rows a norm is folded into the products around it (see parts.OwedRows)
+FOLD_MAX_ROWS = int(os.environ.get("PAE_FOLD_MAX_ROWS", "16"))
+SAME_ORDER_MAX_ROWS = 16  # up to this many rows a product's k ranges depend on its sizes alone
 EPI_BF16, EPI_F32, EPI_SWIGLU, EPI_RESIDUAL = 0, 1, 2, 4
 
 
@@ -520,6 +522,16 @@ def skinny_splits(N: int, K: int, M: int = 1) -> int:
     return -(-K // k_per)
 
 
+_UNITS = 0
+
+
+def _compute_units() -> int:
+    global _UNITS
+    if not _UNITS:
+        _UNITS = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count if torch.cuda.is_available() else 256
+    return _UNITS
+
+
 def residual_splits(N: int, K: int, M: int = 1) -> int:
     """k ranges for a product of up to 16 rows that adds itself into the residual (EPI_RESIDUAL), from
     the product's sizes alone: a row's sums are the same bits whatever it is batched with, launched by
@@ -528,10 +540,18 @@ def residual_splits(N: int, K: int, M: int = 1) -> int:
     workgroups fill the chip or have little to read (1.5B O at 8 rows 7.2 -> 5.9 us, 7B down 38.3 -> 36.1
     us, 72B down 111 -> 107.5 us); a few workgroups with much to read each want ticketed ranges (1.5B
     down: 96 workgroups of 287 KB, 17.4 us in one workgroup each, 12.5 in five ranges)."""
+    if M > SAME_ORDER_MAX_ROWS:
+        return skinny_splits(N, K, M)  # (where norms are folded beyond that many rows: the ranges tuned for the row count)
     tiles = -(-N // 16)
-    if K >= 1024 and (tiles >= 192 or 32 * K <= 65536):
+    # one such workgroup fills a compute unit, so the tiles should fill the chip's units a whole number of
+    # times, or nearly (14B/32B down: 320 tiles are a full round and a quarter of one; 32B at 8 rows 86.7 us
+    # side by side, ticketed ranges are ahead)
+    units = _compute_units()
+    rounds_full = tiles <= units or tiles % units == 0 or tiles % units >= 3 * units // 4
+    if K >= 1024 and (tiles >= 192 or 32 * K <= 65536) and rounds_full:
         return -(-K // (-(-(-(-K // 4)) // 128) * 128))  # four, as the rounding to 128 leaves them
-    return skinny_splits(N, K, 1)
+    splits = skinny_splits(N, K, 1)
+    return splits if splits != 4 else 5 if K // 5 >= 256 else 3  # four would be taken side by side (the same sums, slower here)
 
 
 def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -687,7 +707,7 @@ def whole_sum_splits(N: int, K: int, M: int) -> int:
       14B 37 -> 31 us in four, 72B 87 -> 54 us in six);
     * not with very few weight rows, where the rows of activations are shared out instead."""
     tiles, groups = -(-N // 32), -(-N // 128)
-    if M <= FOLD_MAX_ROWS:
+    if M <= SAME_ORDER_MAX_ROWS:
         # from the sizes alone, so that a row's sums do not depend on the batch (as `residual_splits`).
         # Long rows of weights and not so many of them that the chip is full many times over (the QKV
         # product of the 72B sizes): ranges of about 2,048 (at 8 rows 42.6 -> 40.4 us in four, at one row 39 -> 37 us)
