@@ -38,6 +38,7 @@
 #define PROG_THREADS (PROG_QUADS * 4 * PAE_WAVE)
 #define PROG_MAX_ROWS 16
 #define PROG_SPLIT 128    // keys per split of the attention phase: pae_attn_decode_split()
+#define PROG_STAMPS 8        // clock readings a workgroup may leave per phase in a trace: begin, end, six of the phase's own
 #define PROG_MERGE_ITEMS 256  // (heads of a group) x (head_dim / 4) that one quad merges
 
 struct ProgPhase {
@@ -329,7 +330,7 @@ __device__ __forceinline__ void load_kv_tile_through(bf16x8 (&kf)[HD / 32], s16x
 #define PROG_MERGE_BATCH 16  // splits of one wavefront whose partial results are in flight together
 
 template <int HD>
-__device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad_lds, int* s_flag) {
+__device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad_lds, int* s_flag, long long* stamps) {
   constexpr int TPW = PROG_SPLIT / 64, ROWS = HD / 4 + 2;
   const int lane = threadIdx.x % PAE_WAVE;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE), quad = wave / 4, wq = wave % 4;
@@ -385,6 +386,7 @@ __device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad
         keys_to_mfma_order<HD>(kf[j]);
         if (tile < tile_hi) attn_tile<HD, 1>(st, kf[j], vf[j], qf, tile * 16, pos, start, ph.scale_log2);
       }
+      if (stamps && threadIdx.x == 0 && base == 0) stamps[2] = wall_clock64();
       if (wq > 0) {
         float* mine = quad_lds + (wq - 1) * ROWS * PAE_WAVE;
 #pragma unroll
@@ -437,6 +439,7 @@ __device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad
       }
     }
     if (wq == 0 && lane == 0) s_flag[quad] = to_merge;
+    if (stamps && threadIdx.x == 0 && base == 0) stamps[3] = wall_clock64();
     __syncthreads();
     bool any = false;  // the same in the whole workgroup
 #pragma unroll
@@ -507,6 +510,7 @@ __device__ __forceinline__ void attention_phase(const ProgPhase& ph, float* quad
         put<true>(reinterpret_cast<s16x4*>(ph.attn_out + (int64_t)m_tok * ph.out_stride + (int64_t)(m_kvh * g + c) * HD + d), w);
       }
     }
+    if (stamps && threadIdx.x == 0 && base == 0) stamps[4] = wall_clock64();
     __syncthreads();  // the quads' LDS is free for the next round
   }
 }
@@ -555,15 +559,16 @@ __global__ __launch_bounds__(PROG_THREADS) void decode_program_kernel(const Prog
     const ProgPhase& ph = s_phase[p % 3];
     const ProgPhase* next = p + 1 < num_phases ? &s_phase[(p + 1) % 3] : nullptr;
     if (p + 2 < num_phases) ask_for_phase(p + 2);  // kept when this phase is over
-    if (trace && threadIdx.x == 0) trace[((int64_t)p * gridDim.x + blockIdx.x) * 2] = wall_clock64();
+    if (trace && threadIdx.x == 0) trace[((int64_t)p * gridDim.x + blockIdx.x) * PROG_STAMPS] = wall_clock64();
     if (ph.type == PROG_PRODUCT) {
       product_phase(ph, next, quad_lds, a_lds, parity, ahead);
     } else {
-      if (ph.hd == 128) attention_phase<128>(ph, quad_lds, s_flag);
-      else attention_phase<64>(ph, quad_lds, s_flag);
+      long long* stamps = trace ? trace + ((int64_t)p * gridDim.x + blockIdx.x) * PROG_STAMPS : nullptr;
+      if (ph.hd == 128) attention_phase<128>(ph, quad_lds, s_flag, stamps);
+      else attention_phase<64>(ph, quad_lds, s_flag, stamps);
       ahead = Ahead{};  // nothing is carried across an attention phase (and the registers are free during it)
     }
-    if (trace && threadIdx.x == 0) trace[((int64_t)p * gridDim.x + blockIdx.x) * 2 + 1] = wall_clock64();
+    if (trace && threadIdx.x == 0) trace[((int64_t)p * gridDim.x + blockIdx.x) * PROG_STAMPS + 1] = wall_clock64();
     if (p + 1 == num_phases) break;
     // into the buffer of phase p - 1, whose last readers passed the barrier's workgroup barriers a phase ago
     if (p + 2 < num_phases) keep_phase(p + 2);
@@ -718,7 +723,8 @@ extern "C" int pae_program_max_groups() {
 // `groups` only; `host_error` is an int in pinned host memory that receives 1 + the phase at whose
 // barrier a workgroup gave up after `spin_limit` polls (it stays as it is otherwise).  Launches that
 // share a barrier block or ticket counters must not overlap.  `trace` (or null): device memory for
-// num_phases * groups * 2 clock readings (100 MHz), when every workgroup began and ended every phase.
+// num_phases * groups * 8 clock readings (100 MHz): [0] when the workgroup began the phase, [1] when it ended it,
+// [2..7] marks of the phase's own (attention: every round's items computed, tickets drawn, merges done).
 extern "C" int pae_program_run(const void* phases, int num_phases, void* barrier, int* host_error, int groups,
                                int quad_lds_bytes, int activation_lds_bytes, int spin_limit, long long* trace,
                                hipStream_t stream) {

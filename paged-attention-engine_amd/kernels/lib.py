@@ -393,9 +393,10 @@ class DecodeProgram:
             self._read.record()
 
     def trace_phases(self) -> torch.Tensor:
-        """From now on every launch leaves, per phase and workgroup, the clock (100 MHz) at which it began
-        and ended the phase's work (the difference to the next phase's beginning is its wait at the barrier)."""
-        self.trace = torch.zeros((self.max_phases, self.groups, 2), dtype=torch.int64, device=self.device)
+        """From now on every launch leaves, per phase and workgroup, clock readings (100 MHz): [0] when it
+        began the phase's work, [1] when it ended it (the difference to the next phase's beginning is its
+        wait at the barrier), [2..7] marks of the phase's own (zero where a phase leaves none)."""
+        self.trace = torch.zeros((self.max_phases, self.groups, 8), dtype=torch.int64, device=self.device)
         return self.trace
 
     def check(self) -> None:
