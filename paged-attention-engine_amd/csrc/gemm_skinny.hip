@@ -59,6 +59,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
   float scale[MT];
+  // with one column tile, what the epilogue reads is asked for before the products
+  constexpr bool AHEAD = MT == 1 && (EPI == EPI_RESIDUAL || EPI == EPI_ROPE);
+  EpilogueAhead<RT> ahead;
   const int n0 = blockIdx.x * 16 * RT;
   const int k_lo = (NW == 16 ? wave / 4 : blockIdx.y) * k_per_split;
   const int k_hi = min(K, k_lo + k_per_split);
@@ -139,6 +142,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
     if (kb < k_hi) load(b0, kb);
     // asked for behind the first batch: loads come back in order, so the shares cost no wait of their own
     row_scales<MT>(scale, norm, M, K);
+    if (AHEAD && wave == 0) ask_epilogue<RT, EPI, false>(ahead, blockIdx.x * RT, out, ldc, M, N, rope, norm);
     while (kb < k_hi) {
       if (kb + STEP < k_hi) load(b1, kb + STEP);
       multiply(b0, kb);
@@ -226,7 +230,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
         for (int rt = 0; rt < RT; ++rt) acc[rt][mt] = mine[rt];
   }
   skinny_epilogue<MT, RT, EPI>(acc, blockIdx.x * RT, MT > 1 ? wave : -1, out, ldc, bias, b_is_f32, M, N, blockIdx.y,
-                               part_stride, rope, norm, scale);
+                               part_stride, rope, norm, scale, AHEAD ? &ahead : nullptr);
 }
 
 // The same product for 17..64 rows of A where there are many weight rows.  With several column

@@ -165,6 +165,66 @@ __device__ __forceinline__ void put(short* p, short v) {
   else *p = v;
 }
 
+// What an epilogue reads beside the sums (the residual's tile and the next norm's weights; a row's
+// position, its page of the cache and its angles), asked for before the products are made, so that the
+// trips to memory are over when the sums are there.  One column tile only (up to 16 rows of A).
+template <int RT>
+struct EpilogueAhead {
+  float res[RT][4], next_w[RT][4];  // EPI_RESIDUAL
+  int pos;                          // EPI_ROPE
+  int64_t page;                     //   first element of the row's page in the pools
+  float cs[RT][4][2];               //   cosine and sine of this lane's four features
+};
+
+template <int RT, int EPI, bool THROUGH>
+__device__ __forceinline__ void ask_epilogue(EpilogueAhead<RT>& pre, int tile_base, const void* out, int64_t ldc,
+                                             int M, int N, const SkinnyRope& rope, const SkinnyNorm& norm) {
+  const int lane = threadIdx.x % PAE_WAVE;
+  const int r = lane % 16, g4 = lane / 16;
+  const int mc = r < M ? r : M - 1;
+  if (EPI == EPI_RESIDUAL) {
+    const float* res = (const float*)out + (int64_t)mc * ldc;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int n = 16 * (tile_base + rt) + 4 * g4;
+      if (!THROUGH && ldc % 4 == 0 && n + 4 <= N) {  // the same in the whole wavefront but for the last tile
+        const f32x4 v = *reinterpret_cast<const f32x4*>(res + n);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pre.res[rt][i] = v[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int nc = n + i < N ? n + i : N - 1;
+          pre.res[rt][i] = THROUGH ? load_through(res + nc) : res[nc];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pre.next_w[rt][i] = load_param(norm.next_w, norm.next_w_is_f32, n + i < N ? n + i : N - 1);
+    }
+  }
+  if (EPI == EPI_ROPE) {
+    const int per_head = rope.hd / 16;
+    pre.pos = rope.positions[mc];
+    bool any_cache = false;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int tile = tile_base + rt, head = tile / per_head, j = tile % per_head;
+      any_cache = any_cache || head >= rope.nh;
+      const bool rotated = 16 * j < rope.rot && head < rope.nh + rope.nkv;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float* angle = rope.cos_sin + ((int64_t)mc * (rope.rot / 2) + 8 * j + (4 * g4 + i) % 8) * 2;
+        pre.cs[rt][i][0] = rotated ? angle[0] : 1.f;
+        pre.cs[rt][i][1] = rotated ? angle[1] : 0.f;
+      }
+    }
+    pre.page = 0;
+    if (any_cache)
+      pre.page = (int64_t)rope.block_tables[(int64_t)rope.tok_seq[mc] * rope.max_blocks + pre.pos / rope.bs] *
+                 rope.nkv * ((int64_t)rope.bs * rope.hd);
+  }
+}
+
 // What a wavefront does with finished sums: acc[rt][mt] is the 16 x 16 tile of weight rows
 // 16 (tile_base + rt) .. (through the rotation's row order, if any) by rows 16 mt .. of A; a lane
 // holds row m = 16 mt + lane % 16 of A and weight rows 4 (lane / 16) + i.  only_mt >= 0: just
@@ -174,7 +234,7 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
                                                 void* __restrict__ out, int64_t ldc, const void* __restrict__ bias,
                                                 int b_is_f32, int M, int N, int split, int64_t part_stride,
                                                 const SkinnyRope& rope, const SkinnyNorm& norm,
-                                                const float (&scale)[MT]) {
+                                                const float (&scale)[MT], const EpilogueAhead<RT>* pre = nullptr) {
   const int lane = threadIdx.x % PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
   if (EPI == EPI_ROPE) {
@@ -187,7 +247,7 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
       if (only_mt >= 0 && mt != only_mt) continue;  // another wavefront's column tile
       const int m = 16 * mt + r;
       const int mc = m < M ? m : M - 1;
-      const int pos = rope.positions[mc];
+      const int pos = pre ? pre->pos : rope.positions[mc];
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         const int tile = tile_base + rt;
@@ -205,7 +265,7 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
           float o = own;
           if (rotated) {
             const float* angle = rope.cos_sin + ((int64_t)mc * (rope.rot / 2) + 8 * j + (4 * g4 + i) % 8) * 2;
-            const float cs = angle[0], sn = angle[1];
+            const float cs = pre ? pre->cs[rt][i][0] : angle[0], sn = pre ? pre->cs[rt][i][1] : angle[1];
             o = g4 < 2 ? own * cs - other * sn : own * cs + other * sn;
           }
           res[i] = to_bf16_bits(o);
@@ -216,8 +276,9 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
           continue;
         }
         const int off = pos % rope.bs;
-        const int64_t page = (int64_t)rope.block_tables[(int64_t)rope.tok_seq[m] * rope.max_blocks + pos / rope.bs] *
-                             rope.nkv * head_step;
+        const int64_t page = pre ? pre->page
+                                 : (int64_t)rope.block_tables[(int64_t)rope.tok_seq[m] * rope.max_blocks + pos / rope.bs] *
+                                       rope.nkv * head_step;
         if (head < rope.nh + rope.nkv) {
           put<THROUGH>(reinterpret_cast<s16x4*>(rope.k_cache + page + (head - rope.nh) * head_step + (int64_t)off * rope.hd + f0), res);
         } else {
@@ -266,9 +327,9 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const bool in = n + i < N;
-            v[i] = in ? (THROUGH ? load_through(res + n + i) : res[n + i]) + acc[rt][mt][i] * scale[mt] : 0.f;
+            v[i] = in ? (pre ? pre->res[rt][i] : THROUGH ? load_through(res + n + i) : res[n + i]) + acc[rt][mt][i] * scale[mt] : 0.f;
             ss += v[i] * v[i];
-            p[i] = to_bf16_bits(in ? v[i] * load_param(norm.next_w, norm.next_w_is_f32, n + i) : 0.f);
+            p[i] = to_bf16_bits(in ? v[i] * (pre ? pre->next_w[rt][i] : load_param(norm.next_w, norm.next_w_is_f32, n + i)) : 0.f);
           }
           bf16_t* nxt = norm.next_rows + (int64_t)m * norm.ld_next + n;
           if (vec && norm.ld_next % 4 == 0 && n + 4 <= N) {
@@ -363,13 +424,27 @@ __device__ __forceinline__ bool add_up_k_ranges(f32x4 (&acc)[RT], int slot, int 
   if (lane == 0) __hip_atomic_store(tk.counters + slot, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) acc[rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int p = 0; p < splits; ++p) {
-    const float* theirs = tk.parts + ((int64_t)slot * splits + p) * (RT * 4 * PAE_WAVE) + lane;
+  // added in range order; the loads of four ranges are in flight together (one after the other, every
+  // range would wait out a trip to memory of its own)
+  constexpr int AT_ONCE = RT == 1 ? 4 : RT == 2 ? 2 : 1;  // 16 registers at most
+  for (int p0 = 0; p0 < splits; p0 += AT_ONCE) {
+    float theirs[AT_ONCE][RT * 4];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+    for (int q = 0; q < AT_ONCE; ++q) {
+      const int p = p0 + q < splits ? p0 + q : splits - 1;  // past the last range: loaded again, not added
+      const float* from = tk.parts + ((int64_t)slot * splits + p) * (RT * 4 * PAE_WAVE) + lane;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        acc[rt][i] += __hip_atomic_load(theirs + (rt * 4 + i) * PAE_WAVE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int j = 0; j < RT * 4; ++j)
+        theirs[q][j] = __hip_atomic_load(from + j * PAE_WAVE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int q = 0; q < AT_ONCE; ++q) {
+      if (p0 + q >= splits) break;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[rt][i] += theirs[q][rt * 4 + i];
+    }
   }
   return true;
 }
