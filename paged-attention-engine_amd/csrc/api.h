@@ -82,7 +82,7 @@ int pae_program_put_product_rope(void* phases, int index, void* q_out, int64_t l
 int pae_program_put_attention(void* phases, int index, void* out, int64_t out_stride, const void* q, int64_t q_stride,
                               const void* k_cache, const void* v_cache, const int* dec_work, int num_dec,
                               const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,
-                              int window, void* part_acc, void* part_ml, int* ticket_counters);
+                              int window, void* part_acc, void* part_ml);  // two phases: index and index + 1
 int pae_program_run(const void* phases, int num_phases, void* barrier, int* host_error, int groups, int quad_lds_bytes,
                     int activation_lds_bytes, int spin_limit, long long* trace, hipStream_t stream);
 

@@ -37,6 +37,20 @@ struct SkinnyNorm {
   float* next_stats;       // [M][(N + 15) / 16]
 };
 
+// A pointer that a kernel has read from a description in LDS (not taken as a kernel argument) is a
+// generic one to the compiler: loads through it are flat loads, which count on the LDS counter as well,
+// so that every wait for an LDS read or a cross-lane permute would wait for all of them.  These tell the
+// compiler that such a pointer points into device memory.
+template <typename T>
+__device__ __forceinline__ T* in_memory(T* p) {
+  typedef T __attribute__((address_space(1))) InMemory;
+  InMemory* g = (InMemory*)p;
+  asm("" : "+v"(g));  // hides where it came from: the cast back is then known to come from device memory
+  return (T*)g;
+}
+__device__ __forceinline__ const void* in_memory(const void* p) { return in_memory(reinterpret_cast<const char*>(p)); }
+__device__ __forceinline__ void* in_memory(void* p) { return in_memory(reinterpret_cast<char*>(p)); }
+
 // Loads that see what another die has written through during the same kernel (device-scope loads are
 // served past the die's own L2, which may hold an older copy of the line); see `put` and SkinnyTickets below.
 __device__ __forceinline__ float load_through(const float* p) {
@@ -113,6 +127,15 @@ struct SkinnyRope {
   bf16_t* v_cache;          // [block][kv head][hd][bs]
   int nh, nkv, hd, rot, max_blocks, bs;
 };
+
+__device__ __forceinline__ SkinnyNorm in_memory(const SkinnyNorm& n) {
+  return SkinnyNorm{in_memory(n.row_stats), n.row_stat_tiles, n.eps, in_memory(n.next_rows), n.ld_next,
+                    in_memory(n.next_w), n.next_w_is_f32, in_memory(n.next_stats)};
+}
+__device__ __forceinline__ SkinnyRope in_memory(const SkinnyRope& r) {
+  return SkinnyRope{in_memory(r.cos_sin), in_memory(r.positions), in_memory(r.tok_seq), in_memory(r.block_tables),
+                    in_memory(r.k_cache), in_memory(r.v_cache), r.nh, r.nkv, r.hd, r.rot, r.max_blocks, r.bs};
+}
 
 // Feature within its head of row `r` of the `j`-th tile of a head: a tile inside the rotated
 // part holds features 8 j .. 8 j + 7 (rows 0-7) and their partners rot / 2 + 8 j .. (rows 8-15);

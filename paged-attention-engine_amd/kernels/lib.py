@@ -84,7 +84,7 @@ def _declare(lib) -> None:
         "pae_program_put_product": [P, I, I, P, L, P, L, P, P, I, I, I, I, I, P, P, P, I, F, P, L, P, I, P, P],
         "pae_program_put_product_rope": [P, I, P, L, P, L, P, P, I, I, I, I, I, I, I, P, P, P, P, I, I, P, P, I, P, P, P,
                                          I, F],
-        "pae_program_put_attention": [P, I, P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, P, P, P],
+        "pae_program_put_attention": [P, I, P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, P, P],
         "pae_program_run": [P, I, P, P, I, I, I, I, P, P],
         "pae_program_activation_bytes": [I, I, I],
         "pae_program_lds_limit": [],
@@ -367,13 +367,17 @@ class DecodeProgram:
             self._read.synchronize()  # the launch before has copied the list to the device
         self.count, self.quad_lds, self.activation_lds, self.keep = 0, 0, 0, []
 
+    def room(self, phases: int) -> None:
+        """Raise unless `phases` more fit the list (asked before a pae_program_put_* call writes them)."""
+        if self.count + phases > self.max_phases:
+            raise KernelError(f"a decode program of more than {self.max_phases} phases")
+
     def add(self, code: int, *tensors, activation_bytes: int = 0) -> None:
         """`code`: what a pae_program_put_* call returned (the bytes of LDS a quad needs, or an error);
         `activation_bytes`: the LDS a product's activations take (pae_program_activation_bytes)."""
         if code < 0:
             _check(code)
-        if self.count + 1 > self.max_phases:
-            raise KernelError(f"a decode program of more than {self.max_phases} phases")
+        self.room(1)
         self.count += 1
         self.quad_lds = max(self.quad_lds, code)
         self.activation_lds = max(self.activation_lds, activation_bytes)
@@ -393,9 +397,10 @@ class DecodeProgram:
             self._read.record()
 
     def trace_phases(self) -> torch.Tensor:
-        """From now on every launch leaves, per phase and workgroup, clock readings (100 MHz): [0] when it
-        began the phase's work, [1] when it ended it (the difference to the next phase's beginning is its
-        wait at the barrier), [2..7] marks of the phase's own (zero where a phase leaves none)."""
+        """From now on every launch leaves, per phase and workgroup, eight numbers: clock readings (100 MHz)
+        [0] when it began the phase's work, [1] when it ended it (the difference to the next phase's
+        beginning is its wait at the barrier), [2..5] marks of the phase's own (see pae_program_run; zero
+        where a phase leaves none), and [7] the die that the workgroup ran on."""
         self.trace = torch.zeros((self.max_phases, self.groups, 8), dtype=torch.int64, device=self.device)
         return self.trace
 
@@ -835,14 +840,13 @@ def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cac
     part_acc = torch.empty((n * nh * max_splits, hd), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n * nh * max_splits, 2), dtype=torch.float32, device=q.device)
     if _RECORDING is not None:
-        counters = skinny_tickets(q.device)
-        if n * nkv > counters.numel():
-            raise KernelError(f"{n} tokens by {nkv} key/value heads need more ticket counters than there are")
-        _RECORDING.add(library().pae_program_put_attention(
+        _RECORDING.room(2)  # the splits' partial results, then their merge
+        code = library().pae_program_put_attention(
             _RECORDING.host_ptr, _RECORDING.count, out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
             k_cache.data_ptr(), v_cache.data_ptr(), dec_work.data_ptr(), n, block_tables.data_ptr(),
-            block_tables.shape[1], bs, nh, nkv, hd, float(scale), int(window), part_acc.data_ptr(), part_ml.data_ptr(),
-            counters.data_ptr()), out, q, part_acc, part_ml)
+            block_tables.shape[1], bs, nh, nkv, hd, float(scale), int(window), part_acc.data_ptr(), part_ml.data_ptr())
+        _RECORDING.add(code, out, q, part_acc, part_ml)
+        _RECORDING.add(code)
         return
     _check(library().pae_attn_decode_bf16(
         out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
