@@ -506,6 +506,61 @@ def test_rope_kv_write(dtype, nh, nkv, hd, rot, bs, with_bias):
     assert torch.equal(d_kp.cpu()[untouched], kp[untouched])
 
 
+@pytest.mark.parametrize("nh,nkv,hd,rot,bs", [(12, 2, 128, 128, 16), (6, 1, 48, 48, 16), (3, 3, 32, 16, 8),
+                                              (5, 1, 64, 32, 32), (7, 1, 24, 16, 4), (4, 2, 40, 0, 16)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_rope_kv_write_of_many_rows(nh, nkv, hd, rot, bs, with_bias):
+    """A hundred and more rows of five sequences: portions that begin at a page's first slot, in its
+    middle and at its last slot, a sequence of one token; against the float64 rotation, and bit for bit
+    against the same rows sent 50 at a time (no slot beside the rows' own may change)."""
+    torch.manual_seed(5)
+    theta = 50000.0
+    starts, counts = [0, 5, bs - 1, 3 * bs, 40], [45, 38, 2 * bs + 3, 1, 29]
+    positions, tok_seq = [], []
+    for s, (first, n) in enumerate(zip(starts, counts)):
+        positions += list(range(first, first + n))
+        tok_seq += [s] * n
+    T = len(positions)
+    assert T >= 64 and T % 16 != 0
+    num_blocks = sum(-(-(a + n) // bs) for a, n in zip(starts, counts)) + 5
+    tables = scattered_tables([a + n for a, n in zip(starts, counts)], bs, num_blocks, seed=4)
+    qkv = torch.randn(T, (nh + 2 * nkv) * hd).bfloat16()
+    pos_d = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    seq_d = torch.tensor(tok_seq, dtype=torch.int32, device=DEV)
+    table = K().rope_table(pos_d, plain.rope_inv_freq(rot, theta).to(DEV)) if rot else None
+    kp = torch.full((num_blocks, nkv, bs, hd), 7.0, dtype=torch.bfloat16)
+    vp = torch.full((num_blocks, nkv, hd, bs), 7.0, dtype=torch.bfloat16)
+    bias = torch.randn((nh + 2 * nkv) * hd).bfloat16() if with_bias else None
+    d_bias = bias.to(DEV) if with_bias else None
+    d_qkv, d_kp, d_vp = qkv.to(DEV), kp.to(DEV), vp.to(DEV)
+    K().rope_kv_write(d_qkv, nh, nkv, hd, rot, table, pos_d, seq_d, tables.to(DEV), bs, d_kp, d_vp, d_bias)
+    # the same rows, 50 at a time
+    o_qkv, o_kp, o_vp = qkv.to(DEV), kp.to(DEV), vp.to(DEV)
+    for first in range(0, T, 50):
+        rows = slice(first, min(T, first + 50))
+        K().rope_kv_write(o_qkv[rows], nh, nkv, hd, rot, table[rows] if rot else None, pos_d[rows], seq_d[rows],
+                          tables.to(DEV), bs, o_kp, o_vp, d_bias)
+    assert torch.equal(d_qkv, o_qkv) and torch.equal(d_kp, o_kp) and torch.equal(d_vp, o_vp)
+    ref = (qkv.float() + bias.float()).bfloat16() if with_bias else qkv
+    x = ref.double().view(T, nh + 2 * nkv, hd)
+    rotated = x.clone()
+    if rot:
+        cos, sin = plain.rope_cos_sin(plain.rope_inv_freq(rot, theta, torch.float64), torch.tensor(positions), torch.float64)
+        rotated[..., :rot] = x[..., :rot] * cos[:, None] + plain.rotate_half(x[..., :rot]) * sin[:, None]
+    bound = tol("bfloat16", 4.0)
+    assert (d_qkv.cpu().double().view(T, nh + 2 * nkv, hd)[:, :nh] - rotated[:, :nh]).abs().max() <= bound
+    want_k, want_v = kp.clone().double(), vp.clone().double()
+    untouched_k = torch.ones(num_blocks, bs, dtype=torch.bool)
+    for t, (p, s) in enumerate(zip(positions, tok_seq)):
+        blk = int(tables[s, p // bs])
+        want_k[blk, :, p % bs, :] = rotated[t, nh:nh + nkv]
+        want_v[blk, :, :, p % bs] = x[t, nh + nkv:]
+        untouched_k[blk, p % bs] = False
+    assert (d_kp.cpu().double() - want_k).abs().max() <= bound
+    assert torch.equal(d_vp.cpu().double(), want_v)  # also: no slot beside the rows' own was written
+    assert torch.equal(d_kp.cpu().permute(0, 2, 1, 3)[untouched_k], kp.permute(0, 2, 1, 3)[untouched_k])
+
+
 @pytest.mark.parametrize("M", [1, 7, 16, 23, 64])
 @pytest.mark.parametrize("nh,nkv,hd,rot,bs,Kdim,bias", [
     (4, 2, 16, 16, 4, 72, True), (6, 1, 48, 48, 16, 136, False), (3, 3, 32, 16, 8, 264, True),
