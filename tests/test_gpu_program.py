@@ -88,6 +88,27 @@ def test_a_decode_program_at_the_real_layer_widths_and_sixteen_rows(tmp_path):
     assert runner._eager_program is not None and runner._eager_program.count == 0
 
 
+def test_a_decode_program_whose_wavefronts_take_a_tile_in_several_chunks():
+    """With a width of 2,560 and 6,912 between, a k range is longer than the 14 k steps a wavefront asks
+    for at once (20 for QKV and gate/up, 18 for down's three ranges): a tile's weights then come in two
+    chunks, the next always on the way.  (Wider still, and a range's activations no longer fit LDS beside
+    the attention's: the 7B widths are refused, and run kernel by kernel.)"""
+    wider = dict(WIDE, num_hidden_layers=1, hidden_size=2560, num_attention_heads=20, num_key_value_heads=4,
+                 intermediate_size=6912, vocab_size=1000)
+    model = pae.random_model(wider, seed=4, dtype="bfloat16")
+    for lengths in ((130,), (40, 7, 300, 64, 65, 129, 1, 18, 250)):
+        prompts = [tokens(wider["vocab_size"], n, 31 + n) for n in lengths]
+        alone, cache_alone, _ = run_schedule(model, prompts, 4, use_programs=False)
+        fused, cache_fused, runner = run_schedule(model, prompts, 4, use_programs=True)
+        assert runner._eager_program.count == 6
+        assert torch.equal(fused, alone)
+        assert same_cache(cache_fused, cache_alone)
+    seven_b = dict(wider, hidden_size=3584, num_attention_heads=28, intermediate_size=18944)
+    model = pae.random_model(seven_b, seed=4, dtype="bfloat16")
+    _, _, runner = run_schedule(model, [tokens(1000, 20, 1)], 2, use_programs=True)
+    assert runner._eager_program.count == 0
+
+
 def test_recorded_steps_replay_their_programs(tmp_path):
     """Recorded decode steps hold their program's launch; replays with new tokens, positions and tables
     give what eager steps without programs give, and the oracle's logits within the bound."""
