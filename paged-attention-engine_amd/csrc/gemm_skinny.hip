@@ -241,8 +241,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
 // wants, where every wavefront reads its fragments with one 16-byte read each (two slabs take
 // turns: the next is fetched while the current one is used).  Weight fragments come straight
 // from memory as above.  Every wavefront ends with whole sums of its own rows.
-template <int MT, int RT, int EPI>
-__global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out, int64_t ldc,
+template <int MT, int RT, int EPI, int WAVES = 4>
+__global__ __launch_bounds__(64 * WAVES) void gemm_medium_kernel(void* __restrict__ out, int64_t ldc,
                                                           const bf16_t* __restrict__ A, int64_t lda,
                                                           const bf16_t* __restrict__ W,
                                                           const void* __restrict__ bias, int b_is_f32, int M,
@@ -254,7 +254,8 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
   const int g4 = lane / 16;
   float scale[MT];
   row_scales<MT>(scale, norm, M, K);
-  const int tile_base = (blockIdx.x * 4 + wave) * RT;  // this wavefront's first tile of 16 weight rows
+  const int tile_base = (blockIdx.x * WAVES + wave) * RT;  // this wavefront's first tile of 16 weight rows
+  const bool stages = WAVES == 4 || tid < 256;           // the first four wavefronts bring the slabs of A
   const int k_lo = blockIdx.y * k_per_split;
   const int k_hi = min(K, k_lo + k_per_split);
   const int lrow = lane / 4, lkg = lane % 4;
@@ -290,12 +291,13 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
     bf16x8 wf[KC / 32][RT], a[MT][CH];
   };
   auto load = [&](Slab& b, int kc) {  // loads are unconditional, from clamped addresses
+    if (stages)
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int ka = kc + 128 * c + 8 * achunk;
+      for (int c = 0; c < CH; ++c) {
+        const int ka = kc + 128 * c + 8 * achunk;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) b.a[mt][c] = *reinterpret_cast<const bf16x8*>(aptr[mt] + (ka < K - 8 ? ka : K - 8));
-    }
+        for (int mt = 0; mt < MT; ++mt) b.a[mt][c] = *reinterpret_cast<const bf16x8*>(aptr[mt] + (ka < K - 8 ? ka : K - 8));
+      }
 #pragma unroll
     for (int st = 0; st < KC / 32; ++st) {
       const int k = kc + 32 * st + 8 * lkg;
@@ -304,10 +306,11 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
     }
   };
   auto stage = [&](const Slab& b, int buf) {
+    if (stages)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int c = 0; c < CH; ++c) a_lds[buf][mt][4 * c + a_step][a_slot] = b.a[mt][c];
+        for (int c = 0; c < CH; ++c) a_lds[buf][mt][4 * c + a_step][a_slot] = b.a[mt][c];
   };
   auto multiply = [&](Slab& b, int kc, int buf) {
 #pragma unroll
@@ -350,7 +353,7 @@ __global__ __launch_bounds__(256) void gemm_medium_kernel(void* __restrict__ out
     kc += KC;
   }
   if (EPI != EPI_F32 && tickets.counters) {  // this wavefront's rows: the sums of all k ranges, or done
-    if (!add_up_k_ranges<RT * MT>(reinterpret_cast<f32x4(&)[RT * MT]>(acc), blockIdx.x * 4 + wave, blockIdx.y,
+    if (!add_up_k_ranges<RT * MT>(reinterpret_cast<f32x4(&)[RT * MT]>(acc), blockIdx.x * WAVES + wave, blockIdx.y,
                                   gridDim.y, tickets))
       return;
   }
@@ -401,6 +404,33 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
                     (mt > 3 || (int64_t)medium_groups * splits >= 1024 || (int64_t)narrow_groups * splits < 512);
   // (up to 16 rows every product takes the first kernel, whose order of adding the decode program shares:
   // a row's sums are then the same bits alone, in a batch, in a program or launched by itself)
+  // One k range and 80 weight rows a workgroup (five wavefronts of 16) where that many workgroups are
+  // nearly as many as the chip's 256 compute units: every unit then streams its share of the weights
+  // once, with no partial sums to write and fetch back (1.5B gate/up, 224 workgroups: at 32 rows 19.1 ->
+  // 16.7 us, at 64 rows 23.4 -> 22.2 us against three ticketed ranges of 128-row workgroups; with 205
+  // workgroups, 16,384 weight rows, it is no faster than those).
+  const int groups80 = (N + 79) / 80;
+  if (M > 16 && splits == 1 && groups80 >= 216 && groups80 <= 256 &&
+      (epilogue == EPI_BF16 || epilogue == EPI_F32 || epilogue == EPI_SWIGLU)) {
+#define LAUNCH_80(MT, EPI)                                                                                        \
+  gemm_medium_kernel<MT, 1, EPI, 5><<<dim3(groups80, 1), 320, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
+                                                                        bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets, norm)
+#define BY_MT_80(EPI)                        \
+  switch (mt) {                              \
+    case 2: LAUNCH_80(2, EPI); break;        \
+    case 3: LAUNCH_80(3, EPI); break;        \
+    default: LAUNCH_80(4, EPI); break;       \
+  }
+    switch (epilogue) {
+      case EPI_BF16: BY_MT_80(EPI_BF16); break;
+      case EPI_F32: BY_MT_80(EPI_F32); break;
+      case EPI_SWIGLU: BY_MT_80(EPI_SWIGLU); break;
+      default: return pae_fail("gemm_skinny: epilogue %d has no 80-row form", epilogue);
+    }
+#undef BY_MT_80
+#undef LAUNCH_80
+    return pae_check_launch("gemm_medium (80 rows)");
+  }
   if (M > 16 && ((int64_t)medium_groups * splits >= 256 || only_narrow_fills)) {
     dim3 mgrid(wide ? medium_groups : (N + 63) / 64, splits);
 #define LAUNCH_MEDIUM(MT, EPI)                                                                                   \
