@@ -404,32 +404,41 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
                     (mt > 3 || (int64_t)medium_groups * splits >= 1024 || (int64_t)narrow_groups * splits < 512);
   // (up to 16 rows every product takes the first kernel, whose order of adding the decode program shares:
   // a row's sums are then the same bits alone, in a batch, in a program or launched by itself)
-  // One k range and 80 weight rows a workgroup (five wavefronts of 16) where that many workgroups are
-  // nearly as many as the chip's 256 compute units: every unit then streams its share of the weights
-  // once, with no partial sums to write and fetch back (1.5B gate/up, 224 workgroups: at 32 rows 19.1 ->
-  // 16.7 us, at 64 rows 23.4 -> 22.2 us against three ticketed ranges of 128-row workgroups; with 205
-  // workgroups, 16,384 weight rows, it is no faster than those).
-  const int groups80 = (N + 79) / 80;
-  if (M > 16 && splits == 1 && groups80 >= 216 && groups80 <= 256 &&
-      (epilogue == EPI_BF16 || epilogue == EPI_F32 || epilogue == EPI_SWIGLU)) {
-#define LAUNCH_80(MT, EPI)                                                                                        \
-  gemm_medium_kernel<MT, 1, EPI, 5><<<dim3(groups80, 1), 320, 0, stream>>>(out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, \
-                                                                        bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets, norm)
-#define BY_MT_80(EPI)                        \
-  switch (mt) {                              \
-    case 2: LAUNCH_80(2, EPI); break;        \
-    case 3: LAUNCH_80(3, EPI); break;        \
-    default: LAUNCH_80(4, EPI); break;       \
+  // One k range and 16 W weight rows a workgroup (W = 5 to 8 wavefronts of 16 rows each) where that many
+  // workgroups are nearly as many as the chip's 256 compute units: every unit then streams its share of
+  // the weights once, with no partial sums to write and fetch back (1.5B gate/up, 224 workgroups of 80
+  // rows: at 32 rows 19.1 -> 16.7 us, at 64 rows 23.4 -> 22.2 us against three ticketed ranges of 128-row
+  // workgroups; with 205 workgroups, 16,384 weight rows, it is no faster than those).
+  const int waves = ((N + 15) / 16 + 255) / 256;  // wavefronts a workgroup for at most 256 workgroups
+  const int few_groups = ((N + 15) / 16 + waves - 1) / waves;
+  if (M > 16 && splits == 1 && waves >= 5 && waves <= 8 && few_groups >= 216 &&
+      (epilogue == EPI_BF16 || epilogue == EPI_SWIGLU)) {
+#define LAUNCH_FEW(MT, EPI, W)                                                                                   \
+  gemm_medium_kernel<MT, 1, EPI, W><<<dim3(few_groups, 1), 64 * W, 0, stream>>>(                                  \
+      out, ldc, (const bf16_t*)A, lda, (const bf16_t*)W_, bias, b_is_f32, M, N, K, k_per_split, part_stride, rope, tickets, norm)
+#define FEW_BY_W(MT, EPI)                     \
+  switch (waves) {                            \
+    case 5: LAUNCH_FEW(MT, EPI, 5); break;    \
+    case 6: LAUNCH_FEW(MT, EPI, 6); break;    \
+    case 7: LAUNCH_FEW(MT, EPI, 7); break;    \
+    default: LAUNCH_FEW(MT, EPI, 8); break;   \
   }
-    switch (epilogue) {
-      case EPI_BF16: BY_MT_80(EPI_BF16); break;
-      case EPI_F32: BY_MT_80(EPI_F32); break;
-      case EPI_SWIGLU: BY_MT_80(EPI_SWIGLU); break;
-      default: return pae_fail("gemm_skinny: epilogue %d has no 80-row form", epilogue);
+#define FEW_BY_MT(EPI)                       \
+  switch (mt) {                              \
+    case 2: FEW_BY_W(2, EPI); break;         \
+    case 3: FEW_BY_W(3, EPI); break;         \
+    default: FEW_BY_W(4, EPI); break;        \
+  }
+    const void* W_ = W;
+    if (epilogue == EPI_BF16) {
+      FEW_BY_MT(EPI_BF16);
+    } else {
+      FEW_BY_MT(EPI_SWIGLU);
     }
-#undef BY_MT_80
-#undef LAUNCH_80
-    return pae_check_launch("gemm_medium (80 rows)");
+#undef FEW_BY_MT
+#undef FEW_BY_W
+#undef LAUNCH_FEW
+    return pae_check_launch("gemm_medium (one workgroup a compute unit)");
   }
   if (M > 16 && ((int64_t)medium_groups * splits >= 256 || only_narrow_fills)) {
     dim3 mgrid(wide ? medium_groups : (N + 63) / 64, splits);

@@ -718,9 +718,10 @@ def whole_sum_splits(N: int, K: int, M: int) -> int:
         # Long rows of weights and not so many of them that the chip is full many times over (the QKV
         # product of the 72B sizes): ranges of about 2,048 (at 8 rows 42.6 -> 40.4 us in four, at one row 39 -> 37 us)
         return max(1, min(4, K // 2048)) if N <= 16384 else 1
-    if 216 <= -(-N // 80) <= 256:
-        # one workgroup of 80 weight rows per compute unit, nearly all units busy: one range (the launcher
-        # then takes the five-wavefront kernel; 1.5B gate/up at 32 rows 19.1 -> 16.7 us, at 64 rows 23.4 -> 22.2)
+    waves = -(-(-(-N // 16)) // 256)  # wavefronts of 16 weight rows a workgroup for at most 256 workgroups
+    if 5 <= waves <= 8 and -(-(-(-N // 16)) // waves) >= 216:
+        # one workgroup per compute unit, nearly all units busy: one range (the launcher then takes the
+        # kernel of `waves` wavefronts; 1.5B gate/up at 32 rows 19.1 -> 16.7 us, at 64 rows 23.4 -> 22.2)
         return 1
     if 128 <= groups < 256:
         # a couple of workgroups of 32 weight rows per compute unit: three ranges from 32

@@ -87,7 +87,9 @@ def test_gemm_plain(dtype, M, N, K_):
 
 
 @pytest.mark.parametrize("M", [1, 8, 17, 64])
-@pytest.mark.parametrize("N,K_", [(2048, 1536), (1536, 8960), (50, 72), (777, 64), (96, 200)])
+@pytest.mark.parametrize("N,K_", [(2048, 1536), (1536, 8960), (50, 72), (777, 64), (96, 200),
+                                  # about 256 workgroups of 5, 6, 7 and 8 wavefronts of 16 weight rows (above 16 rows of A)
+                                  (17930, 72), (22000, 136), (27640, 72), (32000, 40)])
 def test_gemm_skinny(M, N, K_):
     torch.manual_seed(M + N)
     a = (torch.randn(M, K_) * 0.5).to(torch.bfloat16)
@@ -107,8 +109,9 @@ def test_gemm_skinny(M, N, K_):
         parts = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device=DEV)
         K().gemm_skinny(parts, a.to(DEV), w.to(DEV), None, K().EPI_F32, splits)
         assert (parts.sum(0).double().cpu() - want).abs().max() <= 2e-5 * scale
-    # a row's result does not depend on the other rows
-    if M > 1:
+    # a row's result does not depend on the other rows (up to 16 rows always; above, where the many
+    # weight rows of the last four shapes do not bring in a kernel that adds k in another order)
+    if M > 1 and (M <= 16 or N < 4096):
         one = torch.empty(1, N, dtype=torch.float32, device=DEV)
         K().gemm_skinny(one, a[M - 1:].to(DEV), w.to(DEV), None, K().EPI_F32)
         assert torch.equal(one[0], out32[M - 1])
@@ -347,7 +350,8 @@ def test_gemm_partial_sums_on_small_workgroups(M):
 
 
 @pytest.mark.parametrize("M", [1, 8, 13, 33, 64])
-@pytest.mark.parametrize("inter,K_", [(8960, 1536), (176, 64), (48, 72), (40, 72), (37888, 136)])
+@pytest.mark.parametrize("inter,K_", [(8960, 1536), (176, 64), (48, 72), (40, 72), (37888, 136),
+                                      (11008, 264), (13824, 136), (16000, 72)])  # workgroups of 6, 7, 8 wavefronts
 def test_gemm_skinny_gated(M, inter, K_):
     torch.manual_seed(inter)
     a = torch.randn(M, K_).to(torch.bfloat16)
