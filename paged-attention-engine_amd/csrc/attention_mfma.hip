@@ -50,6 +50,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   // one load brings the token's row, its position and its table row: a chain of three dependent
   // loads (token, then position and sequence, then pages) would cost a trip to memory each
   const int4 work = dec_work[blockIdx.z];
+  // In a step of single tokens only, token i's sequence is row i of the tables: this wavefront's table
+  // entries are asked for from that row together with the work item, not after it, and used if the
+  // item then names that row (one trip to memory fewer before the keys can be asked for).
+  const int lane = threadIdx.x % PAE_WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE);
+  int guessed[TPW];
+#pragma unroll
+  for (int j = 0; j < TPW; ++j) {
+    const int page = (split * (SPLIT / 16) + wave + 4 * j) * 16 / bs;
+    guessed[j] = block_tables[(int64_t)blockIdx.z * max_blocks + (page < max_blocks ? page : max_blocks - 1)];
+  }
   const int tok = work.x;
   const int pos[1] = {work.y};
   const int start[1] = {(window > 0 && pos[0] - window + 1 > 0) ? pos[0] - window + 1 : 0};
@@ -59,8 +69,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int hi = min((split + 1) * SPLIT, pos[0] + 1);  // keys [lo, hi), not empty
   const int* table = block_tables + (int64_t)work.z * max_blocks;
   const int g = nh / nkv;
-  // (the wavefront's number as a scalar, so that its pages' table entries come by scalar loads)
-  const int lane = threadIdx.x % PAE_WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE);
+  // (the wavefront's number is a scalar, so that its pages' table entries come by scalar loads)
   const int col = lane % 16, g4 = lane / 16;
 
   bf16x8 qf[1][HD / 32];
@@ -88,7 +97,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   for (int j = 0; j < TPW; ++j) {  // a tile past the end is loaded from the first tile's place and not used
     const int tile = tile_lo + wave + 4 * j;
     const int key0 = (tile < tile_hi ? tile : tile_lo) * 16;
-    const int64_t base = ((int64_t)table[key0 / bs] * nkv + kvh) * page_elems;
+    const bool as_guessed = work.z == (int)blockIdx.z && key0 / 16 == split * (SPLIT / 16) + wave + 4 * j;
+    const int64_t base = ((int64_t)(as_guessed ? guessed[j] : table[key0 / bs]) * nkv + kvh) * page_elems;
     load_kv_tile<HD>(kf[j], vf[j], k_cache + base + (int64_t)(key0 % bs) * HD, v_cache + base + key0 % bs, bs);
   }
 #pragma unroll

@@ -841,6 +841,8 @@ def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cac
     assert dec_work.data_ptr() % 16 == 0, "the decode work list must start on a 16-byte boundary"
     n = dec_work.shape[0]
     assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    # (the kernel looks at row i of the tables before it knows token i's own row: the rows must be there)
+    assert n <= block_tables.shape[0], "more single tokens than sequences in the tables"
     max_splits = -(-block_tables.shape[1] * bs // library().pae_attn_decode_split())
     part_acc = torch.empty((n * nh * max_splits, hd), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n * nh * max_splits, 2), dtype=torch.float32, device=q.device)
