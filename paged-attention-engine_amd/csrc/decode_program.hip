@@ -147,9 +147,9 @@ __device__ __forceinline__ bool grid_barrier(ProgBarrier* bar, unsigned& epoch, 
 // are added in wavefront order through LDS, exactly as gemm_skinny_kernel<1, 1, EPI, 4> adds them.
 //
 // Weights do not depend on what a barrier waits for, so a wavefront always has its next chunk of them
-// (up to PROG_S of its k steps, 16 KB a wavefront) on the way: the next tile's while it multiplies the
-// current one, and, across the barrier, those of its first tile of the next phase.  `coming` carries
-// them from one phase to the next.
+// (up to PROG_S of its k steps, 14 KB a wavefront) on the way: the next tile's while it multiplies the
+// current one, and, across the barrier, the first PROG_AHEAD steps of its first tile of the next phase.
+// `coming` carries them from one phase to the next.
 #define PROG_S 14  // most k steps of a wavefront whose weights are asked for together (a chunk)
 #define PROG_AHEAD 4  // steps of its first chunk of the next phase that a wavefront asks for before the barrier
 
@@ -323,7 +323,7 @@ __device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPha
         auto multiply = [&](auto steps) {
 #pragma unroll
           for (int u = 0; u < decltype(steps)::value; ++u) {
-            // four steps' operands at a time (read ahead for all sixteen they would not fit the registers)
+            // four steps' operands at a time (read ahead for a whole chunk they would not fit the registers)
             if (u % 4 == 0 && u > 0) asm volatile("" ::: "memory");
             const int k = kb + 128 * u;  // this wavefront's step: k .. k + 31
             const bool kok = k + 8 * g4 < k_hi;
