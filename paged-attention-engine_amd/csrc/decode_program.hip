@@ -236,7 +236,7 @@ __device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPha
   const int fetch_from = ((lane % 16) * 4 + lane / 16) * 4;
   const bool brief = short_chunks(ph);  // the same in the whole grid
   const int S = brief ? 4 : PROG_S, chunks_a_tile = (steps_of(ph) + S - 1) / S;
-  float scale[1] = {1.0f};
+  float* s_scale = quad_lds + 2 * 3 * 4 * PAE_WAVE;  // [16], behind the two sets of partial sums
   const bf16x8 zero = {};
   const int range_turns = gridDim.x >= splits ? 1 : (splits - blockIdx.x + gridDim.x - 1) / gridDim.x;
   // the quad's chunks of a turn are numbered tile by tile; `in_turn` tells whether chunk j exists and where it lies
@@ -290,7 +290,9 @@ __device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPha
       } else if (!brief) {
         ask_chunk<PROG_S, PROG_AHEAD>(coming, first_chunk);
       }
-      if (wq == 0) row_scales<1, true>(scale, in_memory(ph.norm), M, K);  // behind the weights: they are needed first
+      // what the folded norm owes the rows: the quad's threads together, into the quad's LDS (read after the
+      // barrier that follows the first tile's products)
+      row_scales_to_lds<1, true, 4>(s_scale, in_memory(ph.norm), M, K, threadIdx.x % (4 * PAE_WAVE), [] {});
     }
     const int rounds = (tiles + sh.stride - 1) / sh.stride;  // the same for the quads of a workgroup
     const int total = rounds * chunks_a_tile;
@@ -352,6 +354,7 @@ __device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPha
       for (int w = 0; w < 3; ++w)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[0][0][i] += s_part[(w * 4 + i) * PAE_WAVE + lane];
+      const float scale[1] = {s_scale[lane % 16]};
       if (ph.epilogue != EPI_F32 && splits > 1) {
         f32x4 mine[1] = {acc[0][0]};
         if (!add_up_k_ranges<1>(mine, tile, sh.range, splits, SkinnyTickets{in_memory(ph.ticket_parts), in_memory(ph.ticket_counters)})) continue;
@@ -658,7 +661,7 @@ extern "C" int pae_program_phase_bytes() { return (int)sizeof(ProgPhase); }
 extern "C" int pae_program_barrier_bytes() { return (int)sizeof(ProgBarrier); }
 extern "C" int pae_program_max_rows() { return PROG_MAX_ROWS; }
 
-static int quad_bytes_of_product() { return 2 * 3 * 4 * PAE_WAVE * (int)sizeof(float); }
+static int quad_bytes_of_product() { return (2 * 3 * 4 * PAE_WAVE + 16) * (int)sizeof(float); }
 
 // Bytes of LDS that the activations of one k range of a product take in a workgroup: `rows` rows of one
 // range, whole k steps of 32.

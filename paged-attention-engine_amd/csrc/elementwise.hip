@@ -89,20 +89,18 @@ __global__ void scaled_rows_kernel(bf16_t* __restrict__ out, const bf16_t* __res
   __shared__ float s_scale;
   const int m = blockIdx.x;
   if (threadIdx.x < PAE_WAVE) {
-    // the order in which the products add the shares (gemm_skinny.hip, row_scale_of)
-    const int lane = threadIdx.x, g4 = lane / 16;
+    // the order in which the products of up to 16 rows add the shares (skinny_device.h, row_scales_to_lds):
+    // sixteen threads a row, thread j the groups of four at 4 (16 u + j), one after the other
+    const int j = threadIdx.x % 16;
     const float* shares = row_stats + (int64_t)m * tiles;
     float sum = 0.f;
-    for (int base = 0; base < tiles; base += 128)
-      for (int u = 0; u < 8; ++u) {
-        const int t = base + 16 * u + 4 * g4;
-        float v[4];
-        for (int i = 0; i < 4; ++i) v[i] = t + i < tiles ? shares[t + i] : 0.f;
-        sum += (v[0] + v[1]) + (v[2] + v[3]);
-      }
-    sum += __shfl_xor(sum, 16);
-    sum += __shfl_xor(sum, 32);
-    if (lane == 0) s_scale = rsqrtf(sum / (float)hidden + eps);
+    for (int t = 4 * j; t < tiles; t += 64) {
+      float v[4];
+      for (int i = 0; i < 4; ++i) v[i] = t + i < tiles ? shares[t + i] : 0.f;
+      sum += (v[0] + v[1]) + (v[2] + v[3]);
+    }
+    for (int step = 1; step < 16; step *= 2) sum += __shfl_xor(sum, step);
+    if (threadIdx.x == 0) s_scale = rsqrtf(sum / (float)hidden + eps);
   }
   __syncthreads();
   const float scale = s_scale;

@@ -39,6 +39,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
   // and the trip to memory.
   static_assert(NW == 4 || (NW == 16 && MT == 1), "sixteen wavefronts only with one column tile");
   __shared__ float s_part[MT == 1 ? NW - 1 : 4][RT * MT * 4][PAE_WAVE];
+  __shared__ float s_scale[16 * MT];  // what the folded norm owes every row of A
   if (MT == 1 && gridDim.z > 1) {  // the rows of A are shared out in tiles of 16: this workgroup's tile
     const int m0 = blockIdx.z * 16;
     A += (int64_t)m0 * lda;
@@ -56,9 +57,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
       if (rope.cos_sin) rope.cos_sin += (int64_t)m0 * rope.rot;
     }
   }
-  const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
+  const int tid = threadIdx.x, lane = tid % PAE_WAVE, wave = tid / PAE_WAVE;
   const int r = lane % 16, g4 = lane / 16;
-  float scale[MT];
   // with one column tile, what the epilogue reads is asked for before the products
   constexpr bool AHEAD = MT == 1 && (EPI == EPI_RESIDUAL || EPI == EPI_ROPE);
   EpilogueAhead<RT> ahead;
@@ -133,31 +133,33 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
     }
   };
   constexpr int STEP = KW * SKINNY_U;
-  constexpr bool PIPELINED = true;
   int kb = k_lo + 32 * (wave % 4);  // the same in every lane of a wavefront: the branches on it are uniform
-  if (PIPELINED) {
-    // two batches take turns, so that a wavefront always has loads in flight: with one, every
-    // batch waits out the memory's latency before the next is even asked for
+  {
+    // Two batches take turns, so that a wavefront always has loads in flight: with one, every batch
+    // waits out the memory's latency before the next is even asked for.  No load below stands under a
+    // condition of its own: the compiler counts the loads in flight behind the one it waits for, and
+    // where a load may or may not have been issued it waits for all of them, the other batch's included.
     Batch b0, b1;
-    if (kb < k_hi) load(b0, kb);
-    // asked for behind the first batch: loads come back in order, so the shares cost no wait of their own
-    row_scales<MT>(scale, norm, M, K);
+    int batches = kb < k_hi ? (k_hi - kb + STEP - 1) / STEP : 0;  // of this wavefront
+    // The rows' shares of the sums of squares are asked for first, by the workgroup's first 256 threads
+    // together and all at once, then the first batch (from clamped addresses also where the wavefront
+    // has none); the scales are worked out when the shares are there, with the batch still on its way.
+    row_scales_to_lds<MT>(s_scale, norm, M, K, tid, [&] { load(b0, kb); });
     if (AHEAD && wave == 0) ask_epilogue<RT, EPI, false>(ahead, blockIdx.x * RT, out, ldc, M, N, rope, norm);
-    while (kb < k_hi) {
-      if (kb + STEP < k_hi) load(b1, kb + STEP);
+    while (batches >= 3) {
+      load(b1, kb + STEP);
       multiply(b0, kb);
-      kb += STEP;
-      if (kb >= k_hi) break;
-      if (kb + STEP < k_hi) load(b0, kb + STEP);
-      multiply(b1, kb);
-      kb += STEP;
+      load(b0, kb + 2 * STEP);
+      multiply(b1, kb + STEP);
+      kb += 2 * STEP;
+      batches -= 2;
     }
-  } else {  // more column tiles: the registers go to the activations' fragments
-    row_scales<MT>(scale, norm, M, K);
-    for (; kb < k_hi; kb += STEP) {
-      Batch b;
-      load(b, kb);
-      multiply(b, kb);
+    if (batches == 2) {
+      load(b1, kb + STEP);
+      multiply(b0, kb);
+      multiply(b1, kb + STEP);
+    } else if (batches == 1) {
+      multiply(b0, kb);
     }
   }
 
@@ -215,6 +217,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
       }
   }
 
+  float scale[MT];  // (the barrier above lies between the scales' writing and this)
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) scale[mt] = s_scale[16 * mt + r];
   if (EPI != EPI_F32 && tickets.counters) {  // this wavefront's column tile: the sums of all k ranges, or done
     f32x4 mine[RT];
 #pragma unroll
@@ -250,10 +255,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_medium_kernel(void* __restric
                                                           SkinnyRope rope, SkinnyTickets tickets, SkinnyNorm norm) {
   constexpr int KC = 256 / RT, CH = KC / 128;
   __shared__ bf16x8 a_lds[2][MT][KC / 32][PAE_WAVE];  // [slab][column tile][k step][lane]
+  __shared__ float s_scale[16 * MT];                  // what the folded norm owes every row of A
   const int tid = threadIdx.x, lane = tid % PAE_WAVE, wave = tid / PAE_WAVE;
   const int g4 = lane / 16;
-  float scale[MT];
-  row_scales<MT>(scale, norm, M, K);
   const int tile_base = (blockIdx.x * WAVES + wave) * RT;  // this wavefront's first tile of 16 weight rows
   const bool stages = WAVES == 4 || tid < 256;           // the first four wavefronts bring the slabs of A
   const int k_lo = blockIdx.y * k_per_split;
@@ -330,28 +334,40 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_medium_kernel(void* __restric
       }
     }
   };
-  // the k range is the same for the whole workgroup: every wavefront passes the same barriers
+  // The k range is the same for the whole workgroup: every wavefront passes the same barriers.  Two slabs
+  // take turns; no load stands under a condition of its own (the compiler counts the loads in flight
+  // behind the one it waits for, and where one may or may not have been issued it waits for all).
   Slab s0, s1;
   int kc = k_lo;
-  load(s0, kc);
+  int slabs = (k_hi - k_lo + KC - 1) / KC;  // at least one
+  // the rows' shares of the sums of squares are asked for first, all at once, then the first slab
+  row_scales_to_lds<MT>(s_scale, norm, M, K, tid, [&] { load(s0, kc); });
   stage(s0, 0);
   __syncthreads();
-  while (true) {
-    const bool more0 = kc + KC < k_hi;
-    if (more0) load(s1, kc + KC);
+  while (slabs >= 3) {
+    load(s1, kc + KC);
     multiply(s0, kc, 0);
-    if (!more0) break;
     stage(s1, 1);
     __syncthreads();
-    kc += KC;
-    const bool more1 = kc + KC < k_hi;
-    if (more1) load(s0, kc + KC);
-    multiply(s1, kc, 1);
-    if (!more1) break;
+    load(s0, kc + 2 * KC);
+    multiply(s1, kc + KC, 1);
     stage(s0, 0);
     __syncthreads();
-    kc += KC;
+    kc += 2 * KC;
+    slabs -= 2;
   }
+  if (slabs == 2) {
+    load(s1, kc + KC);
+    multiply(s0, kc, 0);
+    stage(s1, 1);
+    __syncthreads();
+    multiply(s1, kc + KC, 1);
+  } else {
+    multiply(s0, kc, 0);
+  }
+  float scale[MT];  // (written before the first barrier above)
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) scale[mt] = s_scale[16 * mt + lane % 16];
   if (EPI != EPI_F32 && tickets.counters) {  // this wavefront's rows: the sums of all k ranges, or done
     if (!add_up_k_ranges<RT * MT>(reinterpret_cast<f32x4(&)[RT * MT]>(acc), blockIdx.x * WAVES + wave, blockIdx.y,
                                   gridDim.y, tickets))

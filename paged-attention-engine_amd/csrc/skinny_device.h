@@ -73,47 +73,89 @@ __device__ __forceinline__ s16x4 load_through(const s16x4* p) {
   return *reinterpret_cast<s16x4*>(&raw);
 }
 
-// rsqrt(mean of squares + eps) of row m of A from the shares the producer left.  The four lanes
-// that hold row m (g4 = 0..3) read the shares 16 bytes at a time, all reads of a batch of up to
-// 128 shares in flight at once (a loop that adds one share after the other waits out the memory's
-// latency once per share), add theirs in index order and then each other's: the same order in every
-// workgroup, so every column of a row is scaled by the same number.
-template <bool THROUGH = false>
-__device__ __forceinline__ float row_scale_of(const SkinnyNorm& norm, int m, int g4, float inv_width) {
-  const float* shares = norm.row_stats + (int64_t)m * norm.row_stat_tiles;
-  const int tiles = norm.row_stat_tiles;
-  const bool aligned = tiles % 4 == 0;  // rows of shares then start on 16-byte boundaries
-  float sum = 0.f;
-  for (int base = 0; base < tiles; base += 128) {
-    f32x4 part[8];
+// rsqrt(mean of squares + eps) of the rows of A from the shares the producer left, worked out once
+// per workgroup by its first 256 threads together and left in LDS: PER_ROW threads to a row (16 for
+// one column tile, 4 for more), each of which reads every PER_ROW-th group of four shares, all its
+// reads in flight together (a thread that adds up a row in several trips to memory waits out the
+// memory's latency once per trip: with eight trips a wavefront at the 7B width and 64 rows, 18 us a
+// product), adds them in index order, and then the threads of a row add each other's in a fixed
+// order.  The order depends on the width and on MT alone, so every workgroup of a product, and every
+// kernel that takes one column tile, gives a row the same scale.
+template <int MT>
+struct ShareThreads {
+  static constexpr int PER_ROW = MT == 1 ? 16 : 4;
+  static constexpr int AT_ONCE = MT == 1 ? 8 : 16;  // groups of four shares a thread has in flight (up to 512 / 256 shares a row)
+};
+
+// The reads of thread t (0 .. 255 of the workgroup, or of a quad of wavefronts) from `base` on: row t / PER_ROW,
+// the groups of four shares at base + 4 (PER_ROW u + t % PER_ROW), u < AT_ONCE.
+template <int MT, int AT_ONCE, bool THROUGH>
+struct RowShares {
+  f32x4 part[AT_ONCE];
+  __device__ __forceinline__ void ask(const SkinnyNorm& norm, int M, int t, int base) {
+    constexpr int PER_ROW = ShareThreads<MT>::PER_ROW;
+    const int m = t / PER_ROW, j = t % PER_ROW, tiles = norm.row_stat_tiles;
+    const float* shares = norm.row_stats + (int64_t)(m < M ? m : M - 1) * tiles;
+    // Rows of shares start on 16-byte boundaries where tiles % 4 == 0, and a group is then inside a row or
+    // past it as a whole.  (Every group is zeroed first and loaded under one condition of its own: where two
+    // branches load into the same registers the compiler waits for every load in flight in between.)
+    if (tiles % 4 == 0) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int t = base + 16 * u + 4 * g4;
-      if (aligned && t + 4 <= tiles) {
-        part[u] = THROUGH ? load_through(reinterpret_cast<const f32x4*>(shares + t)) : *reinterpret_cast<const f32x4*>(shares + t);
-      } else {
+      for (int u = 0; u < AT_ONCE; ++u) {
+        const int at = base + 4 * (PER_ROW * u + j);
+        part[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (at < tiles)
+          part[u] = THROUGH ? load_through(reinterpret_cast<const f32x4*>(shares + at)) : *reinterpret_cast<const f32x4*>(shares + at);
+      }
+    } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) part[u][i] = t + i < tiles ? (THROUGH ? load_through(shares + t + i) : shares[t + i]) : 0.f;
+      for (int u = 0; u < AT_ONCE; ++u) {
+        const int at = base + 4 * (PER_ROW * u + j);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          part[u][i] = 0.f;
+          if (at + i < tiles) part[u][i] = THROUGH ? load_through(shares + at + i) : shares[at + i];
+        }
       }
     }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) sum += (part[u][0] + part[u][1]) + (part[u][2] + part[u][3]);
   }
-  sum += __shfl_xor(sum, 16);
-  sum += __shfl_xor(sum, 32);
-  return rsqrtf(sum * inv_width + norm.eps);
-}
+  // one group after the other onto `s`: the sum does not depend on how many groups a trip holds
+  __device__ __forceinline__ float add_to(float s) const {
+#pragma unroll
+    for (int u = 0; u < AT_ONCE; ++u) s += (part[u][0] + part[u][1]) + (part[u][2] + part[u][3]);
+    return s;
+  }
+};
 
-// The scales of this lane's rows of A (row 16 mt + lane % 16 of column tile mt), 1 without a folded
-// norm.  Asked for at the start of a kernel, so that the shares arrive while the products run.
-template <int MT, bool THROUGH = false>
-__device__ __forceinline__ void row_scales(float (&scale)[MT], const SkinnyNorm& norm, int M, int K) {
-  const int lane = threadIdx.x % PAE_WAVE;
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = 16 * mt + lane % 16;
-    scale[mt] = norm.row_stats ? row_scale_of<THROUGH>(norm, m < M ? m : M - 1, lane / 16, 1.0f / (float)K) : 1.0f;
+// The scales into s_scale[16 MT] (1 without a folded norm).  Threads t >= 256 do nothing.  The
+// caller puts a workgroup barrier between this and the first read of s_scale.  `before_sum`: called
+// between asking and adding (the place for loads that should be on their way meanwhile).  AT_ONCE:
+// the groups of a trip; fewer cost registers less and wide rows further trips, and give the same bits.
+template <int MT, bool THROUGH = false, int AT_ONCE = ShareThreads<MT>::AT_ONCE, typename Between>
+__device__ __forceinline__ void row_scales_to_lds(float* s_scale, const SkinnyNorm& norm, int M, int K, int t,
+                                                  Between before_sum) {
+  constexpr int PER_ROW = ShareThreads<MT>::PER_ROW;
+  const bool mine = t < 16 * MT * PER_ROW;  // whole wavefronts: 256 threads with one or four column tiles
+  if (!norm.row_stats) {
+    before_sum();
+    if (t < 16 * MT) s_scale[t] = 1.0f;
+    return;
   }
+  const int tiles = norm.row_stat_tiles;
+  constexpr int SPAN = 4 * PER_ROW * AT_ONCE;  // shares of a row that its threads take at once
+  RowShares<MT, AT_ONCE, THROUGH> first;
+  if (mine) first.ask(norm, M, t, 0);
+  before_sum();
+  if (!mine) return;
+  float sum = first.add_to(0.f);
+  for (int base = SPAN; base < tiles; base += SPAN) {  // wider rows: further trips
+    RowShares<MT, AT_ONCE, THROUGH> more;
+    more.ask(norm, M, t, base);
+    sum = more.add_to(sum);
+  }
+#pragma unroll
+  for (int step = 1; step < PER_ROW; step *= 2) sum += __shfl_xor(sum, step);
+  if (t % PER_ROW == 0) s_scale[t / PER_ROW] = rsqrtf(sum / (float)K + norm.eps);
 }
 
 // What the rotating epilogue needs beside the product: the head geometry, the

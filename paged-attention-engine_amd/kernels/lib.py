@@ -436,8 +436,23 @@ class recording:
 
 
 SKINNY_MAX_ROWS = 64
-# up to this many rows a norm is folded into the products around it (see parts.OwedRows)
-FOLD_MAX_ROWS = int(os.environ.get("PAE_FOLD_MAX_ROWS", "16"))
+# Up to this many rows a norm may be folded into the products around it (see parts.OwedRows): as many as
+# the few-rows products take (PAE_FOLD_MAX_ROWS: fewer, for a measurement).  Above 16 rows only while
+# rows x width stays within FOLD_MAX_ELEMENTS: measured at widths 1536 and 3584, folding gains 2.4 to 5 %
+# of the step at 24 to 64 rows of the narrower model and 1.3 / 0.6 % at 24 / 32 rows of the wider, and
+# loses 1.7 / 1.2 % at its 48 / 64 rows, where the norm kernel is cheaper than the products' epilogues
+# that stand in for it.
+FOLD_MAX_ROWS = int(os.environ.get("PAE_FOLD_MAX_ROWS", "64"))
+FOLD_MAX_ELEMENTS = 32 * 3584
+
+
+def folds(rows: int, width: int) -> bool:
+    """Whether a norm of `width` columns is folded into the products around it in a step of `rows` rows."""
+    if not 0 < rows <= FOLD_MAX_ROWS:
+        return False
+    return rows <= SAME_ORDER_MAX_ROWS or rows * width <= FOLD_MAX_ELEMENTS
+
+
 SAME_ORDER_MAX_ROWS = 16  # up to this many rows a product's k ranges depend on its sizes alone
 EPI_BF16, EPI_F32, EPI_SWIGLU, EPI_RESIDUAL = 0, 1, 2, 4
 

@@ -29,8 +29,9 @@ class RMSNorm(Part):
         """(weight, eps) if, in a step of `rows` rows, whatever writes the residual before this norm
         may prepare its rows instead (see `OwedRows`: the consumer's product then pays the scale and
         no norm kernel runs); None if this norm wants to run its own kernel.  The limits are those of
-        the products that pay: bfloat16, few rows, rows of 16-byte multiples."""
-        if self.dtype != torch.bfloat16 or not 0 < rows <= K.FOLD_MAX_ROWS or self.spec.size % 8:
+        the products that pay (bfloat16, few rows, rows of 16-byte multiples) and of where it pays
+        (`kernels.lib.folds`)."""
+        if self.dtype != torch.bfloat16 or not K.folds(rows, self.spec.size) or self.spec.size % 8:
             return None
         return self.weight, self.spec.eps
 

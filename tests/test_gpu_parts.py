@@ -85,8 +85,14 @@ def test_norm_part_and_rows_that_a_product_prepared():
     w_mine, w_other = (1 + 0.1 * torch.randn(width)).bfloat16(), (1 + 0.3 * torch.randn(width)).bfloat16()
     mine.bind("a.", {"a.weight": w_mine})
     other.bind("b.", {"b.weight": w_other})
-    assert mine.folded_for(3) is not None and mine.folded_for(17) is None and mine.folded_for(0) is None
+    from paged_attention_engine_amd.kernels import lib
+    assert mine.folded_for(3) is not None and mine.folded_for(lib.FOLD_MAX_ROWS) is not None
+    assert mine.folded_for(lib.FOLD_MAX_ROWS + 1) is None and mine.folded_for(0) is None
     assert P.build_part(P.NORMS, "norm", spec, torch.float32, DEV).folded_for(3) is None  # float32 runs its kernel
+    # a wide norm is folded at every row count up to 16, above that only while rows x width stays small
+    wide = P.build_part(P.NORMS, "norm", NormSpec(size=lib.FOLD_MAX_ELEMENTS // 32, eps=eps), torch.bfloat16, DEV)
+    wide.bind("c.", {"c.weight": torch.ones(lib.FOLD_MAX_ELEMENTS // 32).bfloat16()})
+    assert wide.folded_for(16) is not None and wide.folded_for(32) is not None and wide.folded_for(33) is None
     res = torch.randn(3, width)
     rows = (res * w_mine.float()).bfloat16()
     stats = torch.zeros(3, K_stat_tiles(width))
