@@ -316,6 +316,7 @@ __device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPha
         acc[0][0] = (f32x4){0.f, 0.f, 0.f, 0.f};
         // what the tile's epilogue reads beside the sums is asked for now (by the wavefront that runs it)
         if (live && wq == 0) {
+          if (ph.epilogue == EPI_ROPE) ask_row<1, EPI_ROPE>(pre, M, in_memory(ph.rope));
           if (ph.epilogue == EPI_ROPE) ask_epilogue<1, EPI_ROPE, false>(pre, tile, nullptr, 0, M, N, in_memory(ph.rope), SkinnyNorm{});
           if (ph.epilogue == EPI_RESIDUAL) ask_epilogue<1, EPI_RESIDUAL, true>(pre, tile, in_memory(ph.out), ph.ldc, M, N, SkinnyRope{}, in_memory(ph.norm));
         }
@@ -357,7 +358,7 @@ __device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPha
       const float scale[1] = {s_scale[lane % 16]};
       if (ph.epilogue != EPI_F32 && splits > 1) {
         f32x4 mine[1] = {acc[0][0]};
-        if (!add_up_k_ranges<1>(mine, tile, sh.range, splits, SkinnyTickets{in_memory(ph.ticket_parts), in_memory(ph.ticket_counters)})) continue;
+        if (!add_up_k_ranges<1, 4>(mine, tile, sh.range, splits, SkinnyTickets{in_memory(ph.ticket_parts), in_memory(ph.ticket_counters)})) continue;
         acc[0][0] = mine[0];
       }
 #define PROG_EPILOGUE(EPI)                                                                                          \

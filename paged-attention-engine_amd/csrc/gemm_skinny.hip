@@ -141,6 +141,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(void* __restrict__
     // where a load may or may not have been issued it waits for all of them, the other batch's included.
     Batch b0, b1;
     int batches = kb < k_hi ? (k_hi - kb + STEP - 1) / STEP : 0;  // of this wavefront
+    if (AHEAD && wave == 0) ask_row<RT, EPI>(ahead, M, rope);
     // The rows' shares of the sums of squares are asked for first, by the workgroup's first 256 threads
     // together and all at once, then the first batch (from clamped addresses also where the wavefront
     // has none); the scales are worked out when the shares are there, with the batch still on its way.
@@ -403,7 +404,10 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   // 72B down 128.5 -> 108.6 us; at 8 rows and below 16 are as fast or faster at most sizes), unless that
   // leaves too few workgroups (the QKV product of the 1.5B sizes at 16 rows: 64 workgroups, 9.2 us)
   const int mt = (M + 15) / 16;
-  const int rt = mt >= 2 || (M > 8 && (int64_t)((N + 31) / 32) * splits >= 128) ? 2 : 1;
+  // (5 to 8 rows with 32 only where there are very many weight rows: 7B gate/up at 8 rows, 1,184 such
+  // workgroups, 59.7 -> 56.3 us; 1.5B gate/up, 560, 11.0 -> 12.2 us)
+  const int64_t groups32 = (int64_t)((N + 31) / 32) * splits;
+  const int rt = mt >= 2 || (M > 8 && groups32 >= 128) || (M > 4 && groups32 >= 1024) ? 2 : 1;
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + 127) / 128 * 128;
   PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "gemm_skinny: %d k ranges are too many for K=%d", splits, K);

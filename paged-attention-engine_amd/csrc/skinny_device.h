@@ -236,11 +236,23 @@ __device__ __forceinline__ void put(short* p, short v) {
 template <int RT>
 struct EpilogueAhead {
   float res[RT][4], next_w[RT][4];  // EPI_RESIDUAL
-  int pos;                          // EPI_ROPE
+  int pos, seq;                     // EPI_ROPE: the row's position and its row of the block tables
   int64_t page;                     //   first element of the row's page in the pools
   float cs[RT][4][2];               //   cosine and sine of this lane's four features
 };
 
+// The part of it that belongs to the row of A alone, and that the page's number waits for: asked for
+// first of all, so that it is there when ask_epilogue wants it.
+template <int RT, int EPI>
+__device__ __forceinline__ void ask_row(EpilogueAhead<RT>& pre, int M, const SkinnyRope& rope) {
+  if (EPI == EPI_ROPE) {
+    const int r = threadIdx.x % 16, mc = r < M ? r : M - 1;
+    pre.pos = rope.positions[mc];
+    pre.seq = rope.nkv > 0 ? rope.tok_seq[mc] : 0;  // (no table without key/value heads)
+  }
+}
+
+// (after ask_row)
 template <int RT, int EPI, bool THROUGH>
 __device__ __forceinline__ void ask_epilogue(EpilogueAhead<RT>& pre, int tile_base, const void* out, int64_t ldc,
                                              int M, int N, const SkinnyRope& rope, const SkinnyNorm& norm) {
@@ -269,7 +281,6 @@ __device__ __forceinline__ void ask_epilogue(EpilogueAhead<RT>& pre, int tile_ba
   }
   if (EPI == EPI_ROPE) {
     const int per_head = rope.hd / 16;
-    pre.pos = rope.positions[mc];
     bool any_cache = false;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
@@ -285,7 +296,7 @@ __device__ __forceinline__ void ask_epilogue(EpilogueAhead<RT>& pre, int tile_ba
     }
     pre.page = 0;
     if (any_cache)
-      pre.page = (int64_t)rope.block_tables[(int64_t)rope.tok_seq[mc] * rope.max_blocks + pre.pos / rope.bs] *
+      pre.page = (int64_t)rope.block_tables[(int64_t)pre.seq * rope.max_blocks + pre.pos / rope.bs] *
                  rope.nkv * ((int64_t)rope.bs * rope.hd);
   }
 }
@@ -470,7 +481,7 @@ struct SkinnyTickets {
 };
 
 // True in the wavefront that holds the whole sums afterwards (in `acc`); the others are done.
-template <int RT>
+template <int RT, int AT_ONCE = (RT == 1 ? 8 : RT == 2 ? 4 : 2)>
 __device__ __forceinline__ bool add_up_k_ranges(f32x4 (&acc)[RT], int slot, int split, int splits,
                                                 const SkinnyTickets& tk) {
   const int lane = threadIdx.x % PAE_WAVE;
@@ -489,9 +500,9 @@ __device__ __forceinline__ bool add_up_k_ranges(f32x4 (&acc)[RT], int slot, int 
   if (lane == 0) __hip_atomic_store(tk.counters + slot, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) acc[rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  // added in range order; the loads of four ranges are in flight together (one after the other, every
-  // range would wait out a trip to memory of its own)
-  constexpr int AT_ONCE = RT == 1 ? 4 : RT == 2 ? 2 : 1;  // 16 registers at most
+  // added in range order; the loads of AT_ONCE ranges are in flight together (one after the other, every
+  // range would wait out a trip to memory of its own: 32 registers by default, which the products' loops
+  // have left free by now, 64 with eight tiles)
   for (int p0 = 0; p0 < splits; p0 += AT_ONCE) {
     float theirs[AT_ONCE][RT * 4];
 #pragma unroll

@@ -562,7 +562,15 @@ def residual_splits(N: int, K: int, M: int = 1) -> int:
     us, 72B down 111 -> 107.5 us); a few workgroups with much to read each want ticketed ranges (1.5B
     down: 96 workgroups of 287 KB, 17.4 us in one workgroup each, 12.5 in five ranges)."""
     if M > SAME_ORDER_MAX_ROWS:
-        return skinny_splits(N, K, M)  # (where norms are folded beyond that many rows: the ranges tuned for the row count)
+        # where norms are folded beyond that many rows: the ranges tuned for the row count, or as many as make
+        # one round of 32-row workgroups over the chip, if those are more and still long (1.5B down at 64 rows:
+        # 48 x 4 workgroups 19.9 us, 48 x 5 17.9 us; at 32 rows 16.8 -> 15.6 us)
+        splits = skinny_splits(N, K, M)
+        one_round = _compute_units() // -(-N // 32)
+        if splits < one_round <= 8 and K // one_round >= 1024:
+            k_per = -(-(-(-K // one_round)) // 128) * 128
+            splits = -(-K // k_per)
+        return splits
     tiles = -(-N // 16)
     # one such workgroup fills a compute unit, so the tiles should fill the chip's units a whole number of
     # times, or nearly (14B/32B down: 320 tiles are a full round and a quarter of one; 32B at 8 rows 86.7 us
