@@ -89,7 +89,9 @@ def test_gemm_plain(dtype, M, N, K_):
 @pytest.mark.parametrize("M", [1, 8, 17, 64])
 @pytest.mark.parametrize("N,K_", [(2048, 1536), (1536, 8960), (50, 72), (777, 64), (96, 200),
                                   # about 256 workgroups of 5, 6, 7 and 8 wavefronts of 16 weight rows (above 16 rows of A)
-                                  (17930, 72), (22000, 136), (27640, 72), (32000, 40)])
+                                  (17930, 72), (22000, 136), (27640, 72), (32000, 40),
+                                  # over a thousand workgroups of 32 weight rows: those already at 8 rows of A
+                                  (33000, 40)])
 def test_gemm_skinny(M, N, K_):
     torch.manual_seed(M + N)
     a = (torch.randn(M, K_) * 0.5).to(torch.bfloat16)
