@@ -554,7 +554,7 @@ def _compute_units() -> int:
 
 
 def residual_splits(N: int, K: int, M: int = 1) -> int:
-    """k ranges for a product of up to 16 rows that adds itself into the residual (EPI_RESIDUAL), from
+    """k ranges for a product that adds itself into the residual (EPI_RESIDUAL).  Up to 16 rows from
     the product's sizes alone: a row's sums are the same bits whatever it is batched with, launched by
     itself or as a phase of a decode program.  Four ranges run side by side in one workgroup of sixteen
     wavefronts, with no tickets and no trip to memory for partial sums, and are ahead wherever the 16-row
