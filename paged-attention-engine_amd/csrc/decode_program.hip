@@ -238,7 +238,8 @@ __device__ __forceinline__ void product_phase(const ProgPhase& ph, const ProgPha
   const int S = brief ? 4 : PROG_S, chunks_a_tile = (steps_of(ph) + S - 1) / S;
   float* s_scale = quad_lds + 2 * 3 * 4 * PAE_WAVE;  // [16], behind the two sets of partial sums
   const bf16x8 zero = {};
-  const int range_turns = gridDim.x >= splits ? 1 : (splits - blockIdx.x + gridDim.x - 1) / gridDim.x;
+  const int groups = (int)gridDim.x, group = (int)blockIdx.x;
+  const int range_turns = groups >= splits ? 1 : (splits - group + groups - 1) / groups;
   // the quad's chunks of a turn are numbered tile by tile; `in_turn` tells whether chunk j exists and where it lies
   auto in_turn = [&](int turn, int j, Chunk& c) -> bool {
     if (turn >= range_turns) return false;

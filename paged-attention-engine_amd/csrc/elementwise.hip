@@ -380,8 +380,6 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, in
   const int t = blockIdx.x;
   const int pos = positions[t];
   T* row = qkv + (int64_t)t * row_stride;
-  const T* k = row + (int64_t)nh * hd;
-  const T* v = k + (int64_t)nkv * hd;
   int64_t page_base = 0;  // element offset of (block, kv head 0) in either pool
   const int64_t head_step = (int64_t)bs * hd;
   const int off = pos % bs;
