@@ -121,7 +121,10 @@ def test_gemm_skinny(M, N, K_):
 
 @pytest.mark.parametrize("M", [1, 8, 12, 17, 40, 64])
 @pytest.mark.parametrize("N,K_,ranges", [(1536, 1536, 4), (1536, 8960, 5), (200, 72, 1), (72, 200, 1), (3584, 512, 2),
-                                          (8192, 1024, 3)])
+                                          (8192, 1024, 3),
+                                          # more shares a row than a workgroup's threads read in one trip (512 with up
+                                          # to 16 rows, 256 above), in whole groups of four and not
+                                          (8256, 64, 1), (8264, 72, 1)])
 def test_a_norm_folded_into_the_products_around_it(M, N, K_, ranges):
     """The product that ends a branch adds itself into the float32 residual and leaves, for the
     product after the next norm, the rows bfloat16(residual * w_norm) and the shares of every
