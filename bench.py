@@ -38,11 +38,20 @@ QWEN25_1P5B = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=28, hid
                    vocab_size=151936, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
                    use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu")
 FULL_LAYERS = 28
-# Other shapes of the same architecture (--model): the 7B and 72B layer sizes, for decode steps and
-# prefills at sizes where a kernel runs longer than a launch costs.
+# Other shapes of the same architecture (--model): the layer sizes of the other Qwen2.5 models, for decode
+# steps and prefills at sizes where a kernel runs longer than a launch costs (7B, 72B) and at the widths in
+# between.
 OTHER_SHAPES = {
+    "0.5b": dict(QWEN25_1P5B, num_hidden_layers=24, hidden_size=896, num_attention_heads=14, num_key_value_heads=2,
+                 head_dim=64, intermediate_size=4864),
+    "3b": dict(QWEN25_1P5B, num_hidden_layers=36, hidden_size=2048, num_attention_heads=16, num_key_value_heads=2,
+               intermediate_size=11008),
     "7b": dict(QWEN25_1P5B, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
                intermediate_size=18944, vocab_size=152064, tie_word_embeddings=False),
+    "14b": dict(QWEN25_1P5B, num_hidden_layers=48, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,
+                intermediate_size=13824, vocab_size=152064, rms_norm_eps=1e-5, tie_word_embeddings=False),
+    "32b": dict(QWEN25_1P5B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,
+                intermediate_size=27648, vocab_size=152064, rms_norm_eps=1e-5, tie_word_embeddings=False),
     "72b": dict(QWEN25_1P5B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
                 num_key_value_heads=8, intermediate_size=29568, vocab_size=152064, rms_norm_eps=1e-5,
                 tie_word_embeddings=False),
@@ -269,7 +278,7 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--ctx", type=int, default=4096)
-    parser.add_argument("--model", choices=("1.5b", "7b", "72b"), default="1.5b",
+    parser.add_argument("--model", choices=("0.5b", "1.5b", "3b", "7b", "14b", "32b", "72b"), default="1.5b",
                         help="layer sizes (default: the Qwen2.5-1.5B shape of the headline figure)")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")

@@ -536,9 +536,16 @@ def skinny_splits(N: int, K: int, M: int = 1) -> int:
             wanted = max(wanted, many)
         # or fewer, longer ranges for that kernel's 64-row workgroups, where those fill the chip and the
         # 128-row ones do not (7B down at 48 rows: 12 ranges 47 us, 8 ranges of 64-row workgroups 42 us)
+        # (ranges down to 768 of k: 14B/32B O, 5,120 x 5,120, at 24 / 64 rows from HBM with the norm: two ranges
+        # 28.2 / 38.0 us, six 22.7 / 27.6)
         fewer = -(-448 // -(-N // 64))
-        if fewer <= 8 and K // fewer >= 1024 and groups * fewer < 256:
+        if fewer <= 8 and K // fewer >= 768 and groups * fewer < 256:
             wanted = fewer
+        # or, with few weight rows, as many ranges as make one round of 32-row workgroups over the chip (3B
+        # down, 64 x 4: 19.9 / 23.7 us with the norm against 23.1 / 29.0 with five ranges; 1.5B down, 48 x 5)
+        one_round = _compute_units() // -(-N // 32)
+        if M > SAME_ORDER_MAX_ROWS and 4 <= one_round <= 8 and K // one_round >= 1024:
+            wanted = one_round
     k_per = -(-(-(-K // wanted)) // 128) * 128
     return -(-K // k_per)
 
@@ -562,15 +569,17 @@ def residual_splits(N: int, K: int, M: int = 1) -> int:
     us, 72B down 111 -> 107.5 us); a few workgroups with much to read each want ticketed ranges (1.5B
     down: 96 workgroups of 287 KB, 17.4 us in one workgroup each, 12.5 in five ranges)."""
     if M > SAME_ORDER_MAX_ROWS:
-        # where norms are folded beyond that many rows: the ranges tuned for the row count, or as many as make
-        # one round of 32-row workgroups over the chip, if those are more and still long (1.5B down at 64 rows:
-        # 48 x 4 workgroups 19.9 us, 48 x 5 17.9 us; at 32 rows 16.8 -> 15.6 us)
-        splits = skinny_splits(N, K, M)
-        one_round = _compute_units() // -(-N // 32)
-        if splits < one_round <= 8 and K // one_round >= 1024:
-            k_per = -(-(-(-K // one_round)) // 128) * 128
-            splits = -(-K // k_per)
-        return splits
+        # Where norms are folded beyond that many rows (all from HBM, at 24 and 64 rows):
+        groups32 = -(-N // 32)
+        if groups32 <= 96 and K <= 6144:
+            # few and short weight rows: one range, no tickets, the rows of A shared out over the workgroups
+            # (0.5B down: 10.7 / 11.2 us against 15.5 / 19.6 in two ticketed ranges and 11.0 / 12.6 in seven)
+            return 1
+        # else the ranges of the partial-sum rule, which suit the residual epilogue as well (1.5B down, 48 x 5
+        # workgroups: 15.6 / 17.9 us against 16.8 / 19.9 with four ranges; 3B down, 64 x 4: 18.5 / 22.9 against
+        # 21.8 / 28.4 with five; 7B down: eight, 35 / 47 us; 14B: six, 33 / 44; 14B O: six, 19 / 27 against 27 / 37
+        # with two)
+        return skinny_splits(N, K, M)
     tiles = -(-N // 16)
     # one such workgroup fills a compute unit, so the tiles should fill the chip's units a whole number of
     # times, or nearly (14B/32B down: 320 tiles are a full round and a quarter of one; 32B at 8 rows 86.7 us
