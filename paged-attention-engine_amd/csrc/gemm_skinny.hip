@@ -405,12 +405,13 @@ static int launch_skinny(int epilogue, void* out, int64_t ldc, const void* A, in
   // sizes), unless that leaves too few workgroups (the QKV product of the 1.5B sizes at 16 rows: 64
   // workgroups, 9.2 us).  5 to 8 rows with 32 only where there are very many weight rows (gate/up at 8
   // rows: 7B, 1,184 such workgroups, 61.1 -> 57.9 us, 32B, 1,728, 129.0 -> 123.2; but 1.5B, 560, 14.2 -> 15.0,
-  // 14B, 864, 67.0 -> 67.6; at 4 rows and below never ahead).  Never with k ranges of 8,192 and more: 72B
+  // 14B, 864, 67.0 -> 67.6; at 4 rows and below never ahead; not with several k ranges: the 72B QKV product
+  // in four ranges, 1,280 such workgroups, 40.4 -> 60.2 us).  Never with k ranges of 8,192 and more: 72B
   // gate/up, whose rows lie 16 KB apart, takes 195.9 us at 9 rows with 16 and 243.9 us with 32.
   const int mt = (M + 15) / 16;
   const int64_t groups32 = (int64_t)((N + 31) / 32) * splits;
   const bool long_ranges = (K + splits - 1) / splits >= 8192;
-  const int rt = mt >= 2 || (!long_ranges && ((M > 8 && groups32 >= 128) || (M > 4 && groups32 >= 1024))) ? 2 : 1;
+  const int rt = mt >= 2 || (!long_ranges && ((M > 8 && groups32 >= 128) || (M > 4 && splits == 1 && groups32 >= 1024))) ? 2 : 1;
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + 127) / 128 * 128;
   PAE_REQUIRE((int64_t)k_per_split * (splits - 1) < K, "gemm_skinny: %d k ranges are too many for K=%d", splits, K);

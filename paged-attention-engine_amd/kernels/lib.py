@@ -516,7 +516,9 @@ def skinny_splits(N: int, K: int, M: int = 1) -> int:
     chip (a workgroup takes 16 weight rows, or 32 and more with more than 8 rows of activations)."""
     rows = 32 if M > 8 else 16
     tiles = -(-N // rows)
-    wanted = max(1, min(512 // tiles, K // 256, 8))
+    # (ranges of at least 1,024 of k: the 0.5B sizes at 8 rows, O 5.3 us in three ranges and 3.9 in one, down
+    # 8.0 us in eight and 7.4 in four)
+    wanted = max(1, min(512 // tiles, K // 1024, 8))
     if M <= 8 and tiles >= 200 and tiles * wanted < 640 and K >= 4096:
         # one or two workgroups per compute unit, each with a long way to go (14B down at 8 rows:
         # 320 workgroups over 13,824 of k take 48 us with the norm, three ranges 35 us)
@@ -589,7 +591,10 @@ def residual_splits(N: int, K: int, M: int = 1) -> int:
     if K >= 1024 and (tiles >= 192 or 32 * K <= 65536) and rounds_full:
         return -(-K // (-(-(-(-K // 4)) // 128) * 128))  # four, as the rounding to 128 leaves them
     splits = skinny_splits(N, K, 1)
-    return splits if splits != 4 else 5 if K // 5 >= 256 else 3  # four would be taken side by side (the same sums, slower here)
+    if splits == 4 and K >= 1024 and (tiles >= 192 or 32 * K <= 65536):
+        # four would be taken side by side (the same sums, slower here)
+        return 5 if K // 5 >= 256 else 3
+    return splits  # (four ticketed ranges where the launcher keeps them apart: 3B down at 8 rows 14.7 us, five 16.5)
 
 
 def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -749,7 +754,8 @@ def whole_sum_splits(N: int, K: int, M: int) -> int:
         # from the sizes alone, so that a row's sums do not depend on the batch (as `residual_splits`).
         # Long rows of weights and not so many of them that the chip is full many times over (the QKV
         # product of the 72B sizes): ranges of about 2,048 (at 8 rows 42.6 -> 40.4 us in four, at one row 39 -> 37 us)
-        return max(1, min(4, K // 2048)) if N <= 16384 else 1
+        # (at the 14B/32B sizes, 5,120 long, one range is ahead: 23.3 / 22.2 us against 24.1 / 23.9 in two)
+        return max(1, min(4, K // 2048)) if N <= 16384 and K >= 8192 else 1
     waves = -(-(-(-N // 16)) // 256)  # wavefronts of 16 weight rows a workgroup for at most 256 workgroups
     if 5 <= waves <= 8 and -(-(-(-N // 16)) // waves) >= 216:
         # one workgroup per compute unit, nearly all units busy: one range (the launcher then takes the
