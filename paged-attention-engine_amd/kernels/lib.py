@@ -751,11 +751,11 @@ def whole_sum_splits(N: int, K: int, M: int) -> int:
     * not with very few weight rows, where the rows of activations are shared out instead."""
     tiles, groups = -(-N // 32), -(-N // 128)
     if M <= SAME_ORDER_MAX_ROWS:
-        # from the sizes alone, so that a row's sums do not depend on the batch (as `residual_splits`).
-        # Long rows of weights and not so many of them that the chip is full many times over (the QKV
-        # product of the 72B sizes): ranges of about 2,048 (at 8 rows 42.6 -> 40.4 us in four, at one row 39 -> 37 us)
-        # (at the 14B/32B sizes, 5,120 long, one range is ahead: 23.3 / 22.2 us against 24.1 / 23.9 in two)
-        return max(1, min(4, K // 2048)) if N <= 16384 and K >= 8192 else 1
+        # from the sizes alone, so that a row's sums do not depend on the batch (as `residual_splits`): one
+        # range at every size (QKV from HBM at 1 / 8 / 16 rows, one range against the best of two to six: 72B
+        # 37.2 / 43.7 / 52.0 us against 36.4 / 42.8 / 59.6; 14B 18.7 / 23.3 / 29.4 against 20.7 / 24.1 / 30.3; 7B 13.1 /
+        # 15.2 / 20.4 against 13.1 / 14.1 / 20.9; gate/up likewise at all seven widths)
+        return 1
     waves = -(-(-(-N // 16)) // 256)  # wavefronts of 16 weight rows a workgroup for at most 256 workgroups
     if 5 <= waves <= 8 and -(-(-(-N // 16)) // waves) >= 216:
         # one workgroup per compute unit, nearly all units busy: one range (the launcher then takes the
@@ -772,7 +772,9 @@ def whole_sum_splits(N: int, K: int, M: int) -> int:
         if K // wanted < 512:
             return 1
     else:
-        wanted = min(8, max(1, (K + 640) // 1280))
+        # (and no more than make about a thousand 32-row workgroups: 72B QKV at 32 / 64 rows, 320 tiles, six
+        # ranges 44.6 / 56.8 us, three 40.3 / 52.9)
+        wanted = min(8, max(1, (K + 640) // 1280), max(1, round(1000 / tiles)))
     k_per = -(-(-(-K // wanted)) // 128) * 128
     return -(-K // k_per)
 
