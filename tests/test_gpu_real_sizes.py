@@ -1,7 +1,8 @@
 """Whole-model logits at the layer sizes the engine is measured at, against the plain implementation.
 
 Two-layer models with the real hidden width, head counts, head size, feed-forward width and
-vocabulary of the Qwen2.5 1.5B, 7B and 72B shapes, random weights drawn on the GPU (the product's
+vocabulary of the Qwen2.5 1.5B, 7B and 72B shapes (and of the 0.5B and 3B shapes, for the replay schedules),
+random weights drawn on the GPU (the product's
 `random_model`; the plain implementation gets the same tensors from the same generator and runs in
 float64 on the GPU as well).  These are the widths at which the serving kernels differ from what
 the tiny models exercise: heads of 128 with 6, 7 and 8 query heads per key/value head in the
@@ -41,6 +42,10 @@ DEV = "cuda:0"
 COMMON = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=2, rope_theta=1000000.0,
               use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu")
 SHAPES = {
+    "0.5b": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, head_dim=64,
+                 intermediate_size=4864, vocab_size=151936, rms_norm_eps=1e-6, tie_word_embeddings=True),
+    "3b": dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=2, head_dim=128,
+               intermediate_size=11008, vocab_size=151936, rms_norm_eps=1e-6, tie_word_embeddings=True),
     "1.5b": dict(hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, head_dim=128,
                  intermediate_size=8960, vocab_size=151936, rms_norm_eps=1e-6, tie_word_embeddings=True),
     "7b": dict(hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, head_dim=128,
@@ -99,8 +104,9 @@ def compare_trace(trace, step_logits, want, dtype, vocab):
     return worst, rms, checked, atol
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", ["1.5b", "7b", "72b"])
+@pytest.mark.parametrize("shape,dtype", [(shape, dtype) for shape in ("1.5b", "7b", "72b") for dtype in ("float32", "bfloat16")]
+                         # the widths in between (other branches of the kernels' rules; heads of 64 at the 0.5B sizes)
+                         + [("0.5b", "float32"), ("0.5b", "bfloat16"), ("3b", "bfloat16")])
 def test_replay_schedules_at_real_layer_sizes(shape, dtype):
     cfg = config_of(shape)
     tokens = request_tokens(cfg, LENGTHS, 11)
