@@ -438,12 +438,13 @@ class recording:
 SKINNY_MAX_ROWS = 64
 # Up to this many rows a norm may be folded into the products around it (see parts.OwedRows): as many as
 # the few-rows products take (PAE_FOLD_MAX_ROWS: fewer, for a measurement).  Above 16 rows only while
-# rows x width stays within FOLD_MAX_ELEMENTS: measured at widths 1536 and 3584, folding gains 2.4 to 5 %
-# of the step at 24 to 64 rows of the narrower model and 1.3 / 0.6 % at 24 / 32 rows of the wider, and
-# loses 1.7 / 1.2 % at its 48 / 64 rows, where the norm kernel is cheaper than the products' epilogues
-# that stand in for it.
+# rows x width stays within FOLD_MAX_ELEMENTS.  Measured with the step itself: folding gains 2 to 6 % at 24
+# to 64 rows of the 0.5B, 1.5B and 3B shapes (widths 896 to 2,048), 1.3 / 0.6 % at 24 / 32 rows of the 7B
+# shape (3,584) and 2.6 % at 24 rows of the 14B shape (5,120), is even at 40 rows of the 7B shape and loses
+# 1.7 / 1.2 % at its 48 / 64 rows, where the norm kernel is cheaper than the products' epilogues that stand
+# in for it.
 FOLD_MAX_ROWS = int(os.environ.get("PAE_FOLD_MAX_ROWS", "64"))
-FOLD_MAX_ELEMENTS = 32 * 3584
+FOLD_MAX_ELEMENTS = 64 * 2048
 
 
 def folds(rows: int, width: int) -> bool:
